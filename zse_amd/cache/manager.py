@@ -18,7 +18,9 @@ prompt up front, cache/cache_manager.py:185-234): ``reserve(req, upto)``
 makes sure every group has pages for positions below ``upto``.
 ``commit(req, n)`` records that n tokens are computed and gives back, in
 windowed groups, each page j with (j+1)*page - 1 <= n - window: its newest key
-is out of sight of every query at position >= n.  ``release(req)`` gives
+is out of sight of every query at position >= n.  In a chunked group (a query
+reads the keys of its own chunk of positions only) it gives back each page whose
+newest key lies before the chunk that position n belongs to.  ``release(req)`` gives
 everything back; a second call does nothing (double free is a no-op,
 cache/cache_manager.py:269-283).
 """
@@ -38,6 +40,19 @@ class GroupInfo:
     window: Optional[int]          # None: keeps every key
     calls: List[int]               # entries of the execution order in this group
     num_pages: int = 0
+    chunk: Optional[int] = None    # keys before the chunk of the next token are never read again
+
+    def first_needed(self, computed: int) -> int:
+        """The first position that a query at position ``computed`` or later can still read."""
+        if self.window is not None:
+            return max(0, computed - self.window + 1)
+        if self.chunk is not None:
+            return computed // self.chunk * self.chunk
+        return 0
+
+    @property
+    def releases(self) -> bool:
+        return self.window is not None or self.chunk is not None
 
 
 @dataclass
@@ -49,14 +64,15 @@ class _Req:
 
 
 def group_needs(needs: Sequence[object]) -> List[GroupInfo]:
-    """Group the paged needs of an execution order by their window."""
+    """Group the paged needs of an execution order by their window (or chunk)."""
     from ..parts.base import PagedKV
-    groups: Dict[Optional[int], GroupInfo] = {}
+    groups: Dict[tuple, GroupInfo] = {}
     for i, n in enumerate(needs):
         if isinstance(n, PagedKV):
-            groups.setdefault(n.window, GroupInfo(n.window, [])).calls.append(i)
-    # windowed groups first, by window; the all-keys group last
-    return sorted(groups.values(), key=lambda g: (g.window is None, g.window or 0))
+            chunk = getattr(n, "chunk", None) if n.window is None else None
+            groups.setdefault((n.window, chunk), GroupInfo(n.window, [], chunk=chunk)).calls.append(i)
+    # windowed groups first, by window; then chunked ones, by chunk; the all-keys group last
+    return sorted(groups.values(), key=lambda g: (g.window is None, g.window or 0, g.chunk is None, g.chunk or 0))
 
 
 class CacheManager:
@@ -138,10 +154,11 @@ class CacheManager:
         ps = self.page_size
         for g, info in enumerate(self.groups):
             out = []
-            if info.window is not None:
+            if info.releases:
                 t = r.tables[g]
                 j = r.first_live[g]
-                while j < len(t) and (j + 1) * ps - 1 <= computed - info.window:
+                first = info.first_needed(computed)
+                while j < len(t) and (j + 1) * ps - 1 < first:
                     if t[j] >= 0:
                         self.pools[g].free(t[j], req)
                         out.append(t[j])
@@ -222,6 +239,6 @@ class CacheManager:
 
     def stats(self) -> dict:
         return {"page_size": self.page_size,
-                "groups": [{"window": g.window, "calls": len(g.calls), "pages": p.num_pages,
+                "groups": [{"window": g.window, "chunk": g.chunk, "calls": len(g.calls), "pages": p.num_pages,
                             "free": p.free_pages} for g, p in zip(self.groups, self.pools)],
                 "live": len(self._reqs), "free_slots": self.slots.free_slots}

@@ -51,6 +51,7 @@ class ShortConvSpec:
     residual: bool = True            # False: the sum alone, without x_t added
     activation: Optional[str] = None  # "silu": applied to the result
     channel_counts: Optional[Tuple[int, ...]] = None   # with several weight names: the channels of each
+    bias: Optional[str] = None       # [size]: where the sum over the taps starts
 
 
 @dataclass(frozen=True)
@@ -65,6 +66,7 @@ class RotarySpec:
     # positions are divided by ``factor``, those that turn more than ``fast`` times stay, a linear
     # ramp over the pair numbers in between; sines and cosines are multiplied by 0.1 ln(factor) + 1
     scaling: Optional[Tuple[float, float, float, float]] = None
+    linear_factor: Optional[float] = None   # every frequency is divided by it (positions stretched); magnitudes stay 1
 
 
 @dataclass(frozen=True)
@@ -95,6 +97,11 @@ class AttentionSpec:
     #                                          channels (pair m by pos * base^(-2m/value_dim)), outputs turned back
     value_pairs_interleaved: bool = False    # pairs (2m, 2m + 1) instead of (m, m + value_dim / 2)
     biases: Optional[Dict[str, str]] = None  # roles q, k, v, o -> names of vectors added in the projections
+    chunk: Optional[int] = None              # keys of the query's own chunk only: floor(i / chunk) == floor(j / chunk),
+    #                                          chunks counted from position 0 of the sequence (not together with window)
+    unit_sink: bool = False                  # a sink of score 0 without a value: weights exp(s_j) / (1 + sum exp(s))
+    qk_unit_norm: bool = False               # q and k divided by their root mean square per head, no gain, AFTER rotation
+    gate: Optional[str] = None               # [num_heads * value_dim, hidden]: heads times sigmoid(W_g x) before W_o
 
 
 @dataclass(frozen=True)
@@ -137,6 +144,48 @@ class DeltaRuleSpec:
 
 
 @dataclass(frozen=True)
+class LinearAttentionSpec:
+    """Gated linear attention: a matrix state per head that decays per key channel,
+    S_t = diag(alpha_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, with q = W_q x key_dim^(-1/2) and
+    alpha = sigmoid(W_a2 (W_a1 x) + b)^(1/tau) (a low-rank projection; decays and state float).
+    The read-out is divided by its root mean square per head, times a gain [value_dim] shared by
+    the heads and silu(W_g x), then W_o."""
+    hidden_size: int
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    decay_rank: int                  # rows of W_a1
+    tau: float
+    eps: float                       # of the read-out's unit RMS
+    names: Dict[str, str]            # roles q, k, v, gate, o, norm, a1, a2, a2_bias
+    kind: str = "gated_linear_attention"
+
+
+@dataclass(frozen=True)
+class SelectiveScanSpec:
+    """A selective scan (Mamba): [u | z] = W_in x; u passes a short causal convolution with bias
+    and silu; [dt | B | C] = W_x u; step = softplus(W_dt dt + b) per channel; A = -exp(A_log);
+    S[c, n] <- exp(step_c A[c, n]) S[c, n] + step_c u_c B_n;  y_c = sum_n S[c, n] C_n + D_c u_c;
+    out = W_o (y silu(z)).  S float [inner, state] per request, beside the convolution's rows."""
+    hidden_size: int
+    inner: int
+    state: int
+    dt_rank: int
+    conv_taps: int
+    names: Dict[str, str]            # roles in, conv, conv_bias, x, dt, dt_bias, A_log, D, o
+    kind: str = "selective_scan"
+
+
+@dataclass(frozen=True)
+class SideBySideSpec:
+    """Several mixers that read the same input; the result is sum_i scales[i] * mixers[i](x).
+    At most one of them keeps pages of keys; their states lie one behind the other."""
+    mixers: Tuple[Any, ...]
+    scales: Tuple[float, ...]
+    kind: str = "side_by_side"
+
+
+@dataclass(frozen=True)
 class MatrixMemorySpec:
     """A recurrent mixer with a matrix state per head (mLSTM): exponential input gate, sigmoid
     forget gate in the log domain, both capped as cap * tanh(x / cap), a running maximum that
@@ -161,6 +210,16 @@ class GatedMLPSpec:
     kind: str = "gated_mlp"
     # clamped_swiglu: g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1)
     limit: Optional[float] = None
+
+
+@dataclass(frozen=True)
+class MLPSpec:
+    """act(x Wu^T), then Wd^T, without a gate.  ``activation``: "relu2" = max(z, 0)^2."""
+    hidden_size: int
+    intermediate_size: int
+    activation: str
+    names: Dict[str, str]            # roles up, down
+    kind: str = "mlp"
 
 
 @dataclass(frozen=True)
@@ -189,15 +248,17 @@ class BlockSpec:
     ``arrangement``:
       "sandwich": h += post_m(mixer(pre_m(h))); h += post_f(ffn(pre_f(h)))
       "prenorm" : h += mixer(pre_m(h));         h += ffn(pre_f(h))
-      "parallel": x = pre_m(h);  h += mixer(x) + ffn(x)      (``ffn`` may be None)
+      "parallel": x = pre_m(h);  h += mixer(x) + ffn(x)      (``ffn`` may be None); with a norm
+                  ``pre_ffn`` among the norms the feed-forward reads pre_f(h) of the same h instead
     ``norms`` holds the roles pre_mixer, post_mixer, pre_ffn, post_ffn that the
-    arrangement uses.
+    arrangement uses.  ``residual_scale`` (parallel): h += residual_scale * (mixer + ffn).
     """
     arrangement: str
     mixer: Any
     ffn: Any
     norms: Dict[str, Any]
     kind: str = "block"
+    residual_scale: float = 1.0
 
 
 @dataclass(frozen=True)

@@ -5,6 +5,10 @@
 //   s_j = softcap((q . k_j) * scale),   j in [lo, pos],  lo = max(0, pos - window + 1)
 //   o   = sum_j softmax(s)_j v_j
 //
+// With ``chunk`` instead of a window, lo = floor(pos / chunk) * chunk: a query sees the keys of
+// its own chunk of positions, counted from position 0.  ``unit_sink``: a sink of score 0 that has
+// no value joins the denominator, exp(s_j) / (1 + sum exp(s)).
+//
 // Keys are visited in tiles of 64 aligned to absolute positions, with a
 // running maximum and sum, so the order of every sum depends on the token's
 // position alone, not on how the step was cut.  Scores, softmax and the output
@@ -26,7 +30,7 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
     const int* __restrict__ req_of_token, const int* __restrict__ positions,
     act_t* __restrict__ out, int nh, int nkv, int hd, int vd, int bs, float scale, float softcap,
     int window, int v_transposed, const float* __restrict__ v_freq, int v_interleaved,
-    const float* __restrict__ sinks, int v_in_k) {
+    const float* __restrict__ sinks, int v_in_k, int chunk, int unit_sink) {
   __shared__ float sq[MAXD];
   __shared__ float sp[64];
   __shared__ int spage[64];
@@ -39,7 +43,7 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
   }
   const int r = req_of_token[t];
   const int kvh = h / (nh / nkv);
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : chunk > 0 ? pos / chunk * chunk : 0;
   const int* table = block_table + (size_t)r * max_blocks;
   const act_t* qr = q + (size_t)t * q_stride + (size_t)h * hd;
   for (int d = lane; d < hd; d += 64) sq[d] = to_f32(qr[d]);
@@ -91,8 +95,8 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
       }
     }
   }
-  if (sinks != nullptr) {
-    const float sk = sinks[h];
+  if (sinks != nullptr || unit_sink) {
+    const float sk = sinks != nullptr ? sinks[h] : 0.f;
     const float m_new = fmaxf(m, sk);
     const float corr = expf(m - m_new);
     l = l * corr + expf(sk - m_new);
@@ -133,12 +137,16 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
 // hd: the size of a head's queries and keys; vd: of its values (the output's too).  v_freq (may
 // be null): float [vd / 2], values are cached turned by their positions and the output is turned back.
 // sinks (may be null): float [nh].  v_in_k: values are the first vd channels of the keys.
-extern "C" int zk_attention_plain_sink(const void* q, int q_stride, const void* kcache, const void* vcache,
-                                       const int* block_table, int max_blocks, const int* req_of_token,
-                                       const int* positions, void* out, int T, int nh, int nkv, int hd, int vd,
-                                       int bs, float scale, float softcap, int window, int v_transposed,
-                                       const float* v_freq, int v_interleaved, const float* sinks, int v_in_k,
-                                       void* stream) {
+// chunk > 0 (without a window): a query sees the keys of its own chunk of positions only.
+// unit_sink: a sink of score 0 joins every head's denominator (not together with sinks).
+extern "C" int zk_attention_plain_masked(const void* q, int q_stride, const void* kcache, const void* vcache,
+                                         const int* block_table, int max_blocks, const int* req_of_token,
+                                         const int* positions, void* out, int T, int nh, int nkv, int hd, int vd,
+                                         int bs, float scale, float softcap, int window, int v_transposed,
+                                         const float* v_freq, int v_interleaved, const float* sinks, int v_in_k,
+                                         int chunk, int unit_sink, void* stream) {
+  ZK_REQUIRE(chunk >= 0 && (chunk == 0 || window <= 0), "zk_attention_plain: a chunk or a window, not both");
+  ZK_REQUIRE(!unit_sink || sinks == nullptr, "zk_attention_plain: a unit sink or learned sinks, not both");
   ZK_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0 && bs > 0 && max_blocks > 0,
              "zk_attention_plain: bad sizes");
   ZK_REQUIRE(vd <= 1024 && (v_freq == nullptr || vd % 2 == 0), "zk_attention_plain: value size above 1024, or odd with a rotation");
@@ -153,13 +161,24 @@ extern "C" int zk_attention_plain_sink(const void* q, int q_stride, const void* 
     attention_plain_kernel<AP_MAX_HD><<<grid, 64, 0, (hipStream_t)stream>>>(
         (const act_t*)q, q_stride, (const act_t*)kcache, (const act_t*)vcache, block_table, max_blocks,
         req_of_token, positions, (act_t*)out, nh, nkv, hd, vd, bs, scale, softcap, window, v_transposed, v_freq,
-        v_interleaved, sinks, v_in_k);
+        v_interleaved, sinks, v_in_k, chunk, unit_sink);
   else
     attention_plain_kernel<1024><<<grid, 64, 0, (hipStream_t)stream>>>(
         (const act_t*)q, q_stride, (const act_t*)kcache, (const act_t*)vcache, block_table, max_blocks,
         req_of_token, positions, (act_t*)out, nh, nkv, hd, vd, bs, scale, softcap, window, v_transposed, v_freq,
-        v_interleaved, sinks, v_in_k);
+        v_interleaved, sinks, v_in_k, chunk, unit_sink);
   return zk_launch_status("zk_attention_plain");
+}
+
+extern "C" int zk_attention_plain_sink(const void* q, int q_stride, const void* kcache, const void* vcache,
+                                       const int* block_table, int max_blocks, const int* req_of_token,
+                                       const int* positions, void* out, int T, int nh, int nkv, int hd, int vd,
+                                       int bs, float scale, float softcap, int window, int v_transposed,
+                                       const float* v_freq, int v_interleaved, const float* sinks, int v_in_k,
+                                       void* stream) {
+  return zk_attention_plain_masked(q, q_stride, kcache, vcache, block_table, max_blocks, req_of_token, positions, out, T,
+                                   nh, nkv, hd, vd, bs, scale, softcap, window, v_transposed, v_freq, v_interleaved,
+                                   sinks, v_in_k, 0, 0, stream);
 }
 
 extern "C" int zk_attention_plain_ext(const void* q, int q_stride, const void* kcache, const void* vcache,
@@ -187,6 +206,9 @@ extern "C" int zk_steplist_register(const char* name, int nargs, void* fn);
 static const int attention_plain_sink_entered = zk_steplist_register(
     "zk_attention_plain_sink", zk_packed::Call<zk_attention_plain_sink>::nargs,
     (void*)zk_packed::Call<zk_attention_plain_sink>::call);
+static const int attention_plain_masked_entered = zk_steplist_register(
+    "zk_attention_plain_masked", zk_packed::Call<zk_attention_plain_masked>::nargs,
+    (void*)zk_packed::Call<zk_attention_plain_masked>::call);
 static const int attention_plain_ext_entered = zk_steplist_register(
     "zk_attention_plain_ext", zk_packed::Call<zk_attention_plain_ext>::nargs,
     (void*)zk_packed::Call<zk_attention_plain_ext>::call);

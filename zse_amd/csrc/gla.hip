@@ -1,0 +1,253 @@
+// Gated linear attention: a recurrent mixer with a matrix state S [D, E] per head whose rows
+// decay each at its own rate.
+//
+//   S <- diag(alpha_t) S + k_t v_t^T;   o_t = S^T q_t
+//
+// with q_t scaled by D^(-1/2), alpha_t = sigmoid(z_t + bias)^(1/tau) = exp(logsigmoid(z_t + bias) / tau)
+// per key channel, and the read-out divided by its root mean square over E, times a gain [E] and
+// silu(g_t).
+//
+// The recurrence never mixes value channels: column e of S and o depends on column e alone.  DS
+// neighbouring lanes own one column of S, each a share of its rows in registers (row chunks of
+// four, dealt out in turn), and walk the tokens of their request; the sum over the rows (S^T q)
+// is joined across the lanes by lane permutations inside the wave, no local memory and no
+// barrier.  q_t, k_t and alpha_t are read from local memory, every column at the same
+// addresses.  Tokens are staged in groups: the block loads q, k of a group and makes its decays,
+// walks it, then norms and gates the group's read-outs (a head whose value channels span several
+// blocks leaves that to a second kernel).  Every sum runs in an order fixed by the channel
+// numbers alone, so a request's values are the same bits however its tokens are cut into steps.
+// All arithmetic is float; q, k, v, g come in the activation type, z as floats.
+#include "common.h"
+#include "packed_call.h"
+
+extern "C" int zk_steplist_register(const char* name, int nargs, void* fn);
+#define ZK_ENTER(fn) \
+  static const int fn##_entered = zk_steplist_register(#fn, zk_packed::Call<fn>::nargs, (void*)zk_packed::Call<fn>::call);
+
+#define GLA_GROUP 16
+#define GLA_COLS 128              // the most value channels a block takes
+#define GLA_COLS_LONG 16          // and what it takes when portions are long: more blocks, a head over more compute units
+
+// The sum of x over the 8 lanes that share a column: lane i with 7 - i, then inside the quads.
+__device__ __forceinline__ float gla_sum8(float x) {
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x141, 0xf, 0xf, false));   // row_half_mirror
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xf, 0xf, false));    // quad_perm [1,0,3,2]
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xf, 0xf, false));    // quad_perm [2,3,0,1]
+  return x;
+}
+__device__ __forceinline__ float gla_sum16(float x) {
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x140, 0xf, 0xf, false));   // row_mirror
+  return gla_sum8(x);
+}
+
+// log(sigmoid(x)) = min(x, 0) - log(1 + exp(-|x|))
+__device__ __forceinline__ float log_sigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
+
+// DS lanes share a column (8 or 16), each holds CH chunks of four rows of S (4 CH DS rows in all, D
+// padded with zeros).  raw (may be null): float [T, H * E], the read-outs before their norm, for a
+// head that spans several blocks.
+template <int CH, int DS>
+__global__ __launch_bounds__(1024) void gla_kernel(
+    const act_t* __restrict__ qkv, int ld, int k_off, int v_off, const act_t* __restrict__ g, int ldg,
+    const float* __restrict__ z, int ldz, const float* __restrict__ z_bias, float inv_tau,
+    const float* __restrict__ gain, float* __restrict__ state, int slot_words, int offset_words,
+    const int* __restrict__ q_start, const int* __restrict__ slot_of_req, act_t* __restrict__ out,
+    float* __restrict__ raw, int H, int D, int E, float eps, float q_scale, int COLS) {
+  constexpr int DMAX = 4 * CH * DS, RD = 4 * CH, GRP = GLA_GROUP;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* qs = lds;                                 // [GRP][DMAX]
+  float* ks = qs + GRP * DMAX;                     // [GRP][DMAX]
+  float* as = ks + GRP * DMAX;                     // [GRP][DMAX]: the decays
+  float* ov = as + GRP * DMAX;                     // [GRP][COLS]: v going in, the read-out coming back
+  const int r = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * COLS, tid = threadIdx.x, nt = blockDim.x;
+  const int lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
+  const int col = tid / DS, j = tid % DS, e = e0 + col;
+  const int t0 = q_start[r], t1 = q_start[r + 1];
+  if (t1 <= t0) return;
+  const bool live = e < E;
+  const int cols = min(COLS, E - e0);
+  float* S = state + (size_t)slot_of_req[r] * slot_words + offset_words + (size_t)h * D * E;
+  float s[RD];
+#pragma unroll
+  for (int i = 0; i < CH; i++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      const int d = 4 * (j + DS * i) + c;
+      s[4 * i + c] = (live && d < D) ? S[(size_t)d * E + e] : 0.f;
+    }
+  for (int c0 = t0; c0 < t1; c0 += GRP) {
+    const int n = min(GRP, t1 - c0);
+    __syncthreads();
+    for (int i = tid; i < n * DMAX; i += nt) {
+      const int tt = i / DMAX, d = i % DMAX;
+      const act_t* row = qkv + (size_t)(c0 + tt) * ld + (size_t)h * D;
+      const bool in = d < D;
+      qs[i] = in ? to_f32(row[d]) * q_scale : 0.f;
+      ks[i] = in ? to_f32(row[k_off + d]) : 0.f;
+      // padding rows of S stay zero whatever their decay
+      as[i] = in ? expf(log_sigmoid_f(z[(size_t)(c0 + tt) * ldz + (size_t)h * D + d] + z_bias[(size_t)h * D + d]) * inv_tau) : 0.f;
+    }
+    for (int i = tid; i < n * COLS; i += nt) {
+      const int tt = i / COLS, c = i % COLS;
+      ov[i] = c < cols ? to_f32(qkv[(size_t)(c0 + tt) * ld + v_off + (size_t)h * E + e0 + c]) : 0.f;
+    }
+    __syncthreads();
+    // the walk: no barrier.  What the next token needs (its k, decays and v) is asked for before this
+    // token's arithmetic.
+    float4 kn[CH], an[CH];
+    float vn;
+    {
+      const float4* k4 = (const float4*)ks + j;
+      const float4* a4 = (const float4*)as + j;
+#pragma unroll
+      for (int i = 0; i < CH; i++) {
+        kn[i] = k4[DS * i];
+        an[i] = a4[DS * i];
+      }
+      vn = ov[col];
+    }
+    for (int tt = 0; tt < n; tt++) {
+      const float4* q4 = (const float4*)(qs + tt * DMAX) + j;
+      const float vt = vn;
+      float4 kk[CH], aa[CH], qq[CH];
+#pragma unroll
+      for (int i = 0; i < CH; i++) {
+        kk[i] = kn[i];
+        aa[i] = an[i];
+        qq[i] = q4[DS * i];
+      }
+      if (tt + 1 < n) {
+        const float4* k4 = (const float4*)(ks + (tt + 1) * DMAX) + j;
+        const float4* a4 = (const float4*)(as + (tt + 1) * DMAX) + j;
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+          kn[i] = k4[DS * i];
+          an[i] = a4[DS * i];
+        }
+        vn = ov[(tt + 1) * COLS + col];
+      }
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+      for (int i = 0; i < CH; i++) {
+        s[4 * i] = fmaf(s[4 * i], aa[i].x, kk[i].x * vt);
+        s[4 * i + 1] = fmaf(s[4 * i + 1], aa[i].y, kk[i].y * vt);
+        s[4 * i + 2] = fmaf(s[4 * i + 2], aa[i].z, kk[i].z * vt);
+        s[4 * i + 3] = fmaf(s[4 * i + 3], aa[i].w, kk[i].w * vt);
+        a0 = fmaf(s[4 * i], qq[i].x, a0);
+        a1 = fmaf(s[4 * i + 1], qq[i].y, a1);
+        a2 = fmaf(s[4 * i + 2], qq[i].z, a2);
+        a3 = fmaf(s[4 * i + 3], qq[i].w, a3);
+      }
+      const float o = DS == 16 ? gla_sum16((a0 + a1) + (a2 + a3)) : gla_sum8((a0 + a1) + (a2 + a3));
+      // a column's v of this token was read (by its lanes, all in one wave) before the read-out
+      // takes its place
+      if (j == 0) ov[tt * COLS + col] = o;
+    }
+    __syncthreads();
+    if (raw != nullptr) {                          // the head spans several blocks: its norm comes later
+      for (int i = tid; i < n * COLS; i += nt) {
+        const int tt = i / COLS, c = i % COLS;
+        if (c < cols) raw[((size_t)(c0 + tt) * H + h) * E + e0 + c] = ov[i];
+      }
+      continue;
+    }
+    for (int tt = wave; tt < n; tt += nw) {        // unit RMS over the head's read-out, gain, gate
+      float ss = 0.f;
+      for (int c = lane; c < E; c += 64) ss = fmaf(ov[tt * COLS + c], ov[tt * COLS + c], ss);
+      ss = wave_sum(ss);
+      const float inv = 1.0f / sqrtf(ss / (float)E + eps);
+      const act_t* gr = g + (size_t)(c0 + tt) * ldg + (size_t)h * E;
+      act_t* orow = out + ((size_t)(c0 + tt) * H + h) * E;
+      for (int c = lane; c < E; c += 64) {
+        const float gg = to_f32(gr[c]);
+        orow[c] = from_f32<act_t>(ov[tt * COLS + c] * inv * gain[c] * (gg / (1.0f + expf(-gg))));
+      }
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < CH; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const int d = 4 * (j + DS * i) + c;
+        if (d < D) S[(size_t)d * E + e] = s[4 * i + c];
+      }
+  }
+}
+
+// One wave per (token, head): out = raw / sqrt(mean(raw^2) + eps) * gain * silu(g).
+__global__ __launch_bounds__(64) void gla_finish_kernel(const float* __restrict__ raw, const act_t* __restrict__ g, int ldg,
+                                                        const float* __restrict__ gain, const int* __restrict__ positions,
+                                                        act_t* __restrict__ out, int H, int E, float eps) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* rr = raw + ((size_t)t * H + h) * E;
+  act_t* orow = out + ((size_t)t * H + h) * E;
+  if (positions[t] < 0) {                          // a padding row of a captured step
+    for (int c = lane; c < E; c += 64) orow[c] = from_f32<act_t>(0.f);
+    return;
+  }
+  float ss = 0.f;
+  for (int c = lane; c < E; c += 64) ss = fmaf(rr[c], rr[c], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)E + eps);
+  const act_t* gr = g + (size_t)t * ldg + (size_t)h * E;
+  for (int c = lane; c < E; c += 64) {
+    const float gg = to_f32(gr[c]);
+    orow[c] = from_f32<act_t>(rr[c] * inv * gain[c] * (gg / (1.0f + expf(-gg))));
+  }
+}
+
+extern "C" {
+
+// qkv: [T, ld] activations: H query heads of D at column 0, H key heads at k_off, H value heads of E
+// at v_off.  g: [T, ldg], H heads of E (the output gate before its silu).  z: float [T, ldz], H heads
+// of D (the decays before bias, sigmoid and root); z_bias: float [H * D]; gain: float [E].
+// state: request r's S [H, D, E] lies at state[slot_of_req[r] * slot_words + offset_words].
+// out: [T, H * E].  Requests are rows [q_start[r], q_start[r + 1]).  raw: float scratch [T, H * E],
+// used by heads that span several blocks (may be null: a head of up to 128 value channels then
+// stays in one block whatever the step); positions: [T].  max_q_len: the longest portion of the
+// step: with long portions a block takes 16 value channels, so that a head's walk spreads over
+// more compute units.
+int zk_gla(const void* qkv, int ld, int k_off, int v_off, const void* g, int ldg, const float* z, int ldz,
+           const float* z_bias, float tau, const float* gain, float* state, int slot_words, int offset_words,
+           const int* q_start, const int* slot_of_req, const int* positions, void* out, float* raw, int T, int R,
+           int max_q_len, int H, int D, int E, float eps, void* stream) {
+  ZK_REQUIRE(T >= 0 && R >= 0 && H > 0 && D > 0 && E > 0 && tau > 0.f, "zk_gla: bad sizes");
+  ZK_REQUIRE(D <= 256, "zk_gla: up to 256 query/key channels a head");
+  ZK_REQUIRE(H <= 65535 && (E + GLA_COLS_LONG - 1) / GLA_COLS_LONG <= 65535, "zk_gla: too many heads or value channels");
+  ZK_REQUIRE(state != nullptr && slot_words >= offset_words + H * D * E, "zk_gla: the state does not fit its slot");
+  ZK_REQUIRE(ldz >= H * D && z != nullptr && z_bias != nullptr, "zk_gla: the decays' rows are too short");
+  const bool scratch = raw != nullptr && positions != nullptr;
+  if (R == 0 || T == 0) return 0;
+  const int DMAX = D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
+  const int DS = DMAX == 256 ? 16 : 8;
+  const bool spread = scratch && max_q_len > GLA_GROUP && E > GLA_COLS_LONG;
+  const int per_block = spread ? GLA_COLS_LONG : DS == 16 ? GLA_COLS / 2 : GLA_COLS;
+  ZK_REQUIRE(E <= per_block || scratch, "zk_gla: a head that spans several blocks needs scratch");
+  const int blocks_e = (E + per_block - 1) / per_block;
+  const int unit = 64 / DS;                                             // columns of a wave
+  const int cols = E < per_block ? (E + unit - 1) / unit * unit : per_block;
+  const int threads = cols * DS;
+  const size_t lds = (size_t)GLA_GROUP * (3 * DMAX + cols) * sizeof(float);
+  dim3 grid(R, H, blocks_e);
+  float* raw_arg = blocks_e > 1 ? raw : nullptr;
+  const float q_scale = 1.0f / sqrtf((float)D);
+#define LAUNCH(C, L)                                                                                              \
+  gla_kernel<C, L><<<grid, threads, lds, (hipStream_t)stream>>>(                                                  \
+      (const act_t*)qkv, ld, k_off, v_off, (const act_t*)g, ldg, z, ldz, z_bias, 1.0f / tau, gain, state,        \
+      slot_words, offset_words, q_start, slot_of_req, (act_t*)out, raw_arg, H, D, E, eps, q_scale, cols)
+  if (DMAX == 32) LAUNCH(1, 8);
+  else if (DMAX == 64) LAUNCH(2, 8);
+  else if (DMAX == 128) LAUNCH(4, 8);
+  else LAUNCH(4, 16);
+#undef LAUNCH
+  if (blocks_e > 1) {
+    dim3 fg(T, H);
+    gla_finish_kernel<<<fg, 64, 0, (hipStream_t)stream>>>(raw, (const act_t*)g, ldg, gain, positions, (act_t*)out, H, E, eps);
+  }
+  return zk_launch_status("zk_gla");
+}
+
+}  // extern "C"
+
+ZK_ENTER(zk_gla)

@@ -23,12 +23,13 @@ __global__ __launch_bounds__(64) void head_prep_kernel(
     const float* __restrict__ q_gain, const float* __restrict__ k_gain, const float* __restrict__ head_scale, float eps,
     const float* __restrict__ inv_freq, int rot_dims, const float* __restrict__ v_freq, int v_interleaved,
     act_t* __restrict__ kcache, act_t* __restrict__ vcache, int nh, int nkv, int D, int E, int bs, int v_transposed,
-    const float* __restrict__ bias, float rot_scale, int qk_interleaved) {
+    const float* __restrict__ bias, float rot_scale, int qk_interleaved, int ld, int unit_norm) {
   __shared__ float buf[HP_MAX];
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int pos = positions[t];
   if (pos < 0) return;                                   // a padding row
-  const size_t width = (size_t)(nh + nkv) * D + (size_t)nkv * E;
+  // ld: the distance between rows where they hold more than the heads (0: just the heads)
+  const size_t width = ld > 0 ? (size_t)ld : (size_t)(nh + nkv) * D + (size_t)nkv * E;
   const int kind = head < nh ? 0 : head < nh + nkv ? 1 : 2;
   const int size = kind == 2 ? E : D;
   const size_t at = (size_t)t * width + (kind == 2 ? (size_t)(nh + nkv) * D + (size_t)(head - nh - nkv) * E : (size_t)head * D);
@@ -71,6 +72,14 @@ __global__ __launch_bounds__(64) void head_prep_kernel(
     buf[ib] = rb;
   }
   __syncthreads();
+  if (unit_norm && kind != 2) {
+    // queries and keys divided by their root mean square over the head, after the rotation, no gain
+    float ss = 0.f;
+    for (int d = lane; d < size; d += 64) ss = fmaf(buf[d], buf[d], ss);
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)size + eps);
+    for (int d = lane; d < size; d += 64) buf[d] *= inv;
+  }
   if (kind == 0) {
     for (int d = lane; d < size; d += 64) qkv[at + d] = from_f32<act_t>(buf[d]);
     return;
@@ -93,11 +102,15 @@ __global__ __launch_bounds__(64) void head_prep_kernel(
 // bias (may be null): float, one per channel of a row, added before anything else.  rot_scale:
 // multiplies the sines and cosines of queries and keys.  qk_interleaved: their pairs are
 // (2i, 2i + 1) instead of (i, i + rot_dims / 2).
-extern "C" int zk_head_prep_ext(void* qkv, const int* positions, const int* slot_map, const float* q_gain,
-                                const float* k_gain, const float* head_scale, float eps, const float* inv_freq,
-                                int rot_dims, const float* v_freq, int v_interleaved, void* kcache, void* vcache, int T,
-                                int nh, int nkv, int D, int E, int bs, int v_transposed, const float* bias,
-                                float rot_scale, int qk_interleaved, void* stream) {
+// ld: the distance between rows of qkv in elements where a row holds more than the heads (0: the
+// heads alone).  unit_norm: queries and keys are divided by their root mean square over the head
+// (with eps), after the rotation and without a gain.
+extern "C" int zk_head_prep_unit(void* qkv, const int* positions, const int* slot_map, const float* q_gain,
+                                 const float* k_gain, const float* head_scale, float eps, const float* inv_freq,
+                                 int rot_dims, const float* v_freq, int v_interleaved, void* kcache, void* vcache, int T,
+                                 int nh, int nkv, int D, int E, int bs, int v_transposed, const float* bias,
+                                 float rot_scale, int qk_interleaved, int ld, int unit_norm, void* stream) {
+  ZK_REQUIRE(ld == 0 || ld >= (nh + nkv) * D + nkv * E, "zk_head_prep: rows shorter than their heads");
   ZK_REQUIRE(T >= 0 && nh > 0 && nkv >= 0 && D > 0 && E > 0 && bs > 0, "zk_head_prep: bad sizes");
   ZK_REQUIRE(D <= HP_MAX && E <= HP_MAX, "zk_head_prep: heads of more than 256 channels are not supported");
   ZK_REQUIRE(inv_freq == nullptr || (rot_dims % 2 == 0 && rot_dims >= 0 && rot_dims <= D),
@@ -110,8 +123,18 @@ extern "C" int zk_head_prep_ext(void* qkv, const int* positions, const int* slot
   head_prep_kernel<<<grid, 64, 0, (hipStream_t)stream>>>((act_t*)qkv, positions, slot_map, q_gain, k_gain, head_scale, eps,
                                                          inv_freq, rot_dims, v_freq, v_interleaved, (act_t*)kcache,
                                                          (act_t*)vcache, nh, nkv, D, E, bs, v_transposed, bias, rot_scale,
-                                                         qk_interleaved);
+                                                         qk_interleaved, ld, unit_norm);
   return zk_launch_status("zk_head_prep");
+}
+
+extern "C" int zk_head_prep_ext(void* qkv, const int* positions, const int* slot_map, const float* q_gain,
+                                const float* k_gain, const float* head_scale, float eps, const float* inv_freq,
+                                int rot_dims, const float* v_freq, int v_interleaved, void* kcache, void* vcache, int T,
+                                int nh, int nkv, int D, int E, int bs, int v_transposed, const float* bias,
+                                float rot_scale, int qk_interleaved, void* stream) {
+  return zk_head_prep_unit(qkv, positions, slot_map, q_gain, k_gain, head_scale, eps, inv_freq, rot_dims, v_freq,
+                           v_interleaved, kcache, vcache, T, nh, nkv, D, E, bs, v_transposed, bias, rot_scale,
+                           qk_interleaved, 0, 0, stream);
 }
 
 extern "C" int zk_head_prep(void* qkv, const int* positions, const int* slot_map, const float* q_gain,
@@ -124,5 +147,7 @@ extern "C" int zk_head_prep(void* qkv, const int* positions, const int* slot_map
 
 static const int head_prep_entered =
     zk_steplist_register("zk_head_prep", zk_packed::Call<zk_head_prep>::nargs, (void*)zk_packed::Call<zk_head_prep>::call);
+static const int head_prep_unit_entered = zk_steplist_register(
+    "zk_head_prep_unit", zk_packed::Call<zk_head_prep_unit>::nargs, (void*)zk_packed::Call<zk_head_prep_unit>::call);
 static const int head_prep_ext_entered = zk_steplist_register(
     "zk_head_prep_ext", zk_packed::Call<zk_head_prep_ext>::nargs, (void*)zk_packed::Call<zk_head_prep_ext>::call);

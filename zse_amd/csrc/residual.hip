@@ -44,6 +44,51 @@ __global__ void sum_norm_kernel(float* __restrict__ h, const void* __restrict__ 
     out[row + i] = from_f32<act_t>(hr[i] * inv * (unit_offset ? 1.0f + w_next[i] : w_next[i]));
 }
 
+// h <- h + mult * (a + b + bias); out1 = norm(h) * gain1, out2 = norm(h) * gain2: a layer whose two
+// sublayers read two norms of the same stream (either output may be absent)
+__global__ void sum_norm_pair_kernel(float* __restrict__ h, const void* __restrict__ a, int a_parts,
+                                     const void* __restrict__ b, int b_parts, const float* __restrict__ bias, float mult,
+                                     const float* __restrict__ w1, act_t* __restrict__ out1,
+                                     const float* __restrict__ w2, act_t* __restrict__ out2, float eps, int unit_offset,
+                                     int W) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const size_t plane = (size_t)gridDim.x * W, row = (size_t)r * W;
+  float* hr = h + row;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v = hr[i];
+    if (a != nullptr || b != nullptr || bias != nullptr) {
+      float y = planes_value(a, a_parts, plane, row + i) + planes_value(b, b_parts, plane, row + i);
+      if (bias) y += bias[i];
+      v = fmaf(mult, y, v);
+      hr[i] = v;
+    }
+    ss = fmaf(v, v, ss);
+  }
+  if (!w1 && !w2) return;
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {      // each thread re-reads what it wrote
+    const float x = hr[i] * inv;
+    if (w1) out1[row + i] = from_f32<act_t>(x * (unit_offset ? 1.0f + w1[i] : w1[i]));
+    if (w2) out2[row + i] = from_f32<act_t>(x * (unit_offset ? 1.0f + w2[i] : w2[i]));
+  }
+}
+
+// out[t, :] = sum_i scale_i x_i[t, :] as one float plane; the terms are activations
+__global__ void weighted_sum_kernel(const act_t* __restrict__ x0, float s0, const act_t* __restrict__ x1, float s1,
+                                    const act_t* __restrict__ x2, float s2, const act_t* __restrict__ x3, float s3,
+                                    float* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float y = s0 * to_f32(x0[i]);
+  if (x1) y = fmaf(s1, to_f32(x1[i]), y);
+  if (x2) y = fmaf(s2, to_f32(x2[i]), y);
+  if (x3) y = fmaf(s3, to_f32(x3[i]), y);
+  out[i] = y;
+}
+
 // y[t, :] += bias
 __global__ void add_bias_kernel(act_t* __restrict__ y, const float* __restrict__ bias, int W) {
   const size_t row = (size_t)blockIdx.x * W;
@@ -71,6 +116,32 @@ int zk_sum_norm(float* h, const void* a, int a_parts, const void* b, int b_parts
   return zk_launch_status("zk_sum_norm");
 }
 
+// As zk_sum_norm, with the sublayers' sum times ``mult`` and up to two norms of the new stream
+// (w1 -> out1, w2 -> out2; either pair may be null).  a, b and bias all null: the stream stays as
+// it is and only the norms are made.
+int zk_sum_norm_pair(float* h, const void* a, int a_parts, const void* b, int b_parts, const float* bias, float mult,
+                     const float* w1, void* out1, const float* w2, void* out2, float eps, int unit_offset, int T, int W,
+                     void* stream) {
+  ZK_REQUIRE(T >= 0 && W > 0 && a_parts >= 0 && b_parts >= 0, "zk_sum_norm_pair: bad sizes");
+  ZK_REQUIRE((w1 == nullptr || out1 != nullptr) && (w2 == nullptr || out2 != nullptr), "zk_sum_norm_pair: a norm without output");
+  if (T == 0) return 0;
+  const int threads = (ZSE_ACT_BF16 && T <= 64 && W >= 1024) ? 1024 : 256;
+  sum_norm_pair_kernel<<<T, threads, 0, (hipStream_t)stream>>>(h, a, a_parts, b, b_parts, bias, mult, w1, (act_t*)out1, w2,
+                                                              (act_t*)out2, eps, unit_offset, W);
+  return zk_launch_status("zk_sum_norm_pair");
+}
+
+// out (float [T, W]) = s0 x0 + s1 x1 + s2 x2 + s3 x3 over activations [T, W]; x1..x3 may be null.
+int zk_weighted_sum(const void* x0, float s0, const void* x1, float s1, const void* x2, float s2, const void* x3, float s3,
+                    float* out, int T, int W, void* stream) {
+  ZK_REQUIRE(T >= 0 && W > 0 && x0 != nullptr && out != nullptr, "zk_weighted_sum: bad arguments");
+  if (T == 0) return 0;
+  const size_t n = (size_t)T * W;
+  weighted_sum_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+      (const act_t*)x0, s0, (const act_t*)x1, s1, (const act_t*)x2, s2, (const act_t*)x3, s3, out, n);
+  return zk_launch_status("zk_weighted_sum");
+}
+
 int zk_add_bias(void* y, const float* bias, int T, int W, void* stream) {
   ZK_REQUIRE(T >= 0 && W > 0 && bias != nullptr, "zk_add_bias: bad sizes");
   if (T == 0) return 0;
@@ -88,5 +159,7 @@ int zk_planes_sum(const float* planes, int parts, void* out, int T, int W, void*
 }  // extern "C"
 
 ZK_ENTER(zk_sum_norm)
+ZK_ENTER(zk_sum_norm_pair)
+ZK_ENTER(zk_weighted_sum)
 ZK_ENTER(zk_add_bias)
 ZK_ENTER(zk_planes_sum)

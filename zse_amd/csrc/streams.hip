@@ -138,7 +138,7 @@ __global__ void short_conv_kernel(const act_t* __restrict__ h, const float* __re
                                   int slot_words, int offset_words, const int* __restrict__ positions,
                                   const int* __restrict__ req_of_token, const int* __restrict__ q_start,
                                   const int* __restrict__ slot_of_req, act_t* __restrict__ out, int W, int taps,
-                                  int ld_in, int ld_out, int residual, int act) {
+                                  int ld_in, int ld_out, int residual, int act, const float* __restrict__ bias) {
   const int t = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= W) return;
@@ -150,7 +150,7 @@ __global__ void short_conv_kernel(const act_t* __restrict__ h, const float* __re
   const int before = t - q_start[r];      // rows of this step in front of t that belong to the same request
   float* st = state + (size_t)slot_of_req[r] * slot_words + offset_words;
   const float x = to_f32(h[(size_t)t * ld_in + c]);
-  float acc = 0.f;
+  float acc = bias ? bias[c] : 0.f;
   for (int j = 0; j < taps; j++) {
     const int back = taps - 1 - j;
     float v;
@@ -256,9 +256,10 @@ int zk_streams_step(float* xs, int S, const void* y, int y_parts, const float* w
 // [W, taps]; the state of request r is taps - 1 float rows of W at
 // state[slot_of_req[r] * slot_words + offset_words].  residual: the input is added to the sum;
 // act: 0 none, 1 silu (after the sum).
-int zk_short_conv_ext(const void* h, int ld_in, const float* w, const float* state, int slot_words, int offset_words,
-                      const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
-                      void* out, int ld_out, int T, int W, int taps, int residual, int act, void* stream) {
+int zk_short_conv_bias(const void* h, int ld_in, const float* w, const float* state, int slot_words, int offset_words,
+                       const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
+                       void* out, int ld_out, int T, int W, int taps, int residual, int act, const float* bias,
+                       void* stream) {
   ZK_REQUIRE(T >= 0 && T <= 65535 * 16 && W > 0 && taps >= 1, "zk_short_conv: bad sizes");
   ZK_REQUIRE(ld_in >= W && ld_out >= W && (act == 0 || act == 1), "zk_short_conv: bad strides or activation");
   ZK_REQUIRE(taps == 1 || (state != nullptr && slot_words >= offset_words + (taps - 1) * W),
@@ -268,8 +269,16 @@ int zk_short_conv_ext(const void* h, int ld_in, const float* w, const float* sta
   dim3 grid((W + 255) / 256, T);
   short_conv_kernel<false><<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)h, w, (float*)state, slot_words, offset_words,
                                                                   positions, req_of_token, q_start, slot_of_req,
-                                                                  (act_t*)out, W, taps, ld_in, ld_out, residual, act);
+                                                                  (act_t*)out, W, taps, ld_in, ld_out, residual, act, bias);
   return zk_launch_status("zk_short_conv");
+}
+
+// bias (zk_short_conv_bias; may be null): float [W], where the sum over the taps starts.
+int zk_short_conv_ext(const void* h, int ld_in, const float* w, const float* state, int slot_words, int offset_words,
+                      const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
+                      void* out, int ld_out, int T, int W, int taps, int residual, int act, void* stream) {
+  return zk_short_conv_bias(h, ld_in, w, state, slot_words, offset_words, positions, req_of_token, q_start, slot_of_req, out,
+                            ld_out, T, W, taps, residual, act, nullptr, stream);
 }
 
 int zk_short_conv(const void* h, const float* w, const float* state, int slot_words, int offset_words,
@@ -281,9 +290,10 @@ int zk_short_conv(const void* h, const float* w, const float* state, int slot_wo
 
 // The convolution and the renewal of the state in one launch, for steps in which every request
 // brings exactly one token (T rows, T requests).
-int zk_short_conv_token_ext(const void* h, int ld_in, const float* w, float* state, int slot_words, int offset_words,
-                            const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
-                            void* out, int ld_out, int T, int W, int taps, int residual, int act, void* stream) {
+int zk_short_conv_token_bias(const void* h, int ld_in, const float* w, float* state, int slot_words, int offset_words,
+                             const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
+                             void* out, int ld_out, int T, int W, int taps, int residual, int act, const float* bias,
+                             void* stream) {
   ZK_REQUIRE(T >= 0 && T <= 65535 && W > 0 && taps >= 1, "zk_short_conv_token: bad sizes");
   ZK_REQUIRE(ld_in >= W && ld_out >= W && (act == 0 || act == 1), "zk_short_conv_token: bad strides or activation");
   ZK_REQUIRE(taps == 1 || (state != nullptr && slot_words >= offset_words + (taps - 1) * W),
@@ -292,8 +302,15 @@ int zk_short_conv_token_ext(const void* h, int ld_in, const float* w, float* sta
   dim3 grid((W + 255) / 256, T);
   short_conv_kernel<true><<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)h, w, state, slot_words, offset_words, positions,
                                                                  req_of_token, q_start, slot_of_req, (act_t*)out, W, taps,
-                                                                 ld_in, ld_out, residual, act);
+                                                                 ld_in, ld_out, residual, act, bias);
   return zk_launch_status("zk_short_conv_token");
+}
+
+int zk_short_conv_token_ext(const void* h, int ld_in, const float* w, float* state, int slot_words, int offset_words,
+                            const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
+                            void* out, int ld_out, int T, int W, int taps, int residual, int act, void* stream) {
+  return zk_short_conv_token_bias(h, ld_in, w, state, slot_words, offset_words, positions, req_of_token, q_start,
+                                  slot_of_req, out, ld_out, T, W, taps, residual, act, nullptr, stream);
 }
 
 int zk_short_conv_token(const void* h, const float* w, float* state, int slot_words, int offset_words,
@@ -338,6 +355,8 @@ ZK_ENTER(zk_short_conv)
 ZK_ENTER(zk_short_conv_token)
 ZK_ENTER(zk_short_conv_state)
 ZK_ENTER(zk_short_conv_ext)
+ZK_ENTER(zk_short_conv_bias)
+ZK_ENTER(zk_short_conv_token_bias)
 ZK_ENTER(zk_short_conv_token_ext)
 ZK_ENTER(zk_short_conv_state_ext)
 ZK_ENTER(zk_rotate_heads)

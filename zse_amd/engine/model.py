@@ -116,6 +116,8 @@ class Model:
         from ..parts.norm import RMSNorm
         norm = blk.entry_norm() if hasattr(blk, "entry_norm") else None
         T, H = h.shape
+        if isinstance(out, tuple):
+            out = out[0]
         if isinstance(norm, RMSNorm):
             ns = norm.spec
             ctx.k.zk_sum_norm(h.ptr, first.ptr, 1, None, 0, None, norm.weight.ptr, float(ns.eps), int(ns.unit_offset),
@@ -135,6 +137,9 @@ class Model:
         # its output alternates between two buffers that outlive a layer's own
         T, H = h.shape
         handoff = [ctx.alloc((T, H)), ctx.alloc((T, H))]
+        if any(isinstance(b.entry_norm(), tuple) for b in self.blocks if hasattr(b, "entry_norm")):
+            # a block that reads two norms of the stream at once gets both from the block before
+            handoff = [(t, ctx.alloc((T, H))) for t in handoff]
         # an order that adds the embedding's output to the stream again keeps a copy of it
         again = any(getattr(c, "add_embedding", False) for c in order)
         # (gathered a second time: a launch like any other, which a captured or written-down step repeats)
@@ -151,7 +156,10 @@ class Model:
                 x = self._add_embedding(ctx, h, first, blk, handoff[(i + 1) % 2])
             if hasattr(blk, "entry_norm"):
                 next_norm = nxt.entry_norm() if nxt is not None and hasattr(nxt, "entry_norm") else None
-                x = blk.forward(ctx, h, cache, x_in=x, next_norm=next_norm, x_out=handoff[i % 2])
+                out = handoff[i % 2]
+                if isinstance(out, tuple) and not isinstance(next_norm, tuple):
+                    out = out[0]
+                x = blk.forward(ctx, h, cache, x_in=x, next_norm=next_norm, x_out=out)
             else:
                 blk.forward(ctx, h, cache)
                 x = None

@@ -197,6 +197,10 @@ class StepRunner:
                     shape = (pages, need.num_kv_heads, vd, self.page_size)
                 # values that are part of the keys have no slab of their own
                 cc.v = cc.k if getattr(need, "values_in_keys", False) else rt.zeros(shape, self.dtype)
+                if getattr(need, "state_bytes", 0):      # a mixer that keeps a state beside its pages
+                    cc.state_offset = slot_bytes
+                    cc.state_bytes = int(need.state_bytes)
+                    slot_bytes += (int(need.state_bytes) + 15) // 16 * 16
             elif isinstance(need, StateNeed):
                 cc.state_offset = slot_bytes
                 cc.state_bytes = int(need.nbytes)

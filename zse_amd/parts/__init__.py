@@ -1,5 +1,6 @@
 """Parts a model is put together from.  Importing the package registers the built-in kinds."""
-from . import attention, block, delta, embedding, ffn, latent, mlstm, norm, position, shortconv, streams  # noqa: F401
+from . import (attention, block, delta, embedding, ffn, gla, latent, mlstm, norm, position, scan, shortconv,  # noqa: F401
+               sidebyside, streams)
 from .base import (PagedKV, Part, StateNeed, TensorReq, build_part, register_part,
                    unregister_part, walk)
 from ..runtime.device import register_kernels  # noqa: F401  (a part that brings kernels of its own)

@@ -17,7 +17,7 @@ from typing import List
 
 import numpy as np
 
-from ..runtime.device import BF16, Tensor
+from ..runtime.device import BF16, ITEMSIZE, Tensor
 from .base import ROLE_GAIN, PagedKV, Part, TensorReq, build_part, register_part
 from .ops import linear, tuned_gemm
 
@@ -43,9 +43,18 @@ class PagedAttention(Part):
         self.bias_names = dict(getattr(s, "biases", None) or {})
         self.rot_scale = float(self.position.magnitude()) if hasattr(self.position, "magnitude") else 1.0
         self.rot_interleaved = bool(getattr(self.position, "interleaved", False))
+        self.chunk = int(getattr(s, "chunk", None) or 0)
+        self.unit_sink = bool(getattr(s, "unit_sink", False))
+        self.unit_norm = bool(getattr(s, "qk_unit_norm", False))
+        self.gate_name = getattr(s, "gate", None)
+        if self.chunk and s.window:
+            raise ValueError("an attention has a window or a chunk, not both")
+        if self.chunk < 0:
+            raise ValueError(f"chunk must be positive, got {self.chunk}")
         self.general = bool(self.value_dim != s.head_dim or self.q_norm_name or self.k_norm_name or
                             self.head_scale_name or self.value_base or self.bias_names or
-                            self.rot_scale != 1.0 or self.rot_interleaved)
+                            self.rot_scale != 1.0 or self.rot_interleaved or self.chunk or self.unit_sink or
+                            self.unit_norm or self.gate_name)
         self.in_bias = self.o_bias = None
         if self.value_dim > 256:
             raise ValueError(f"value_dim up to 256, got {self.value_dim}")
@@ -65,6 +74,8 @@ class PagedAttention(Part):
             out.append(TensorReq(self.q_norm_name, (s.head_dim,), ROLE_GAIN))
         if self.head_scale_name:
             out.append(TensorReq(self.head_scale_name, (s.num_heads,), ROLE_GAIN))
+        if self.gate_name:
+            out.append(TensorReq(self.gate_name, (s.num_heads * self.value_dim, s.hidden_size)))
         for role, rows in (("q", s.num_heads * s.head_dim), ("o", s.hidden_size)):
             if role in self.bias_names:
                 out.append(TensorReq(self.bias_names[role], (rows,), ROLE_GAIN))
@@ -82,6 +93,8 @@ class PagedAttention(Part):
     def load(self, weights, rt, dtype):
         s = self.spec
         names = [s.names["q"]] if self.shared_kv else [s.names[r] for r in ("q", "k", "v")]
+        if self.gate_name:
+            names.append(self.gate_name)       # the gate's rows behind q, k, v: one product
         strip = getattr(weights, "wants_strip", None)
         self.w_qkv = weights.matrix(names, strip=True) if strip and strip(s.hidden_size) else weights.matrix(names)
         o_cols = s.num_heads * self.value_dim
@@ -107,7 +120,7 @@ class PagedAttention(Part):
     def cache_need(self):
         s = self.spec
         return PagedKV(s.num_kv_heads, s.head_dim, s.window,
-                       self.value_dim if self.value_dim != s.head_dim else None)
+                       self.value_dim if self.value_dim != s.head_dim else None, chunk=self.chunk or None)
 
     def flops_per_key(self) -> float:
         return 2.0 * self.spec.num_heads * (self.spec.head_dim + self.value_dim)        # q.k and p.v
@@ -117,6 +130,8 @@ class PagedAttention(Part):
     def wants_v_transposed(self, kernels, dtype: str, page_size: int) -> bool:
         """The matrix-core kernel reads V as [page][kv head][hd][bs]."""
         s = self.spec
+        if (self.chunk or self.unit_sink) and not kernels.has("zk_attention_bf16_masked"):
+            return False
         return bool(dtype == BF16 and self.value_dim == s.head_dim and kernels.has("zk_attention_bf16") and
                     kernels.zk_attention_bf16_supports(s.num_heads, s.num_kv_heads, s.head_dim, page_size))
 
@@ -162,7 +177,8 @@ class PagedAttention(Part):
         T = x.shape[0]
         nh, nkv, hd, vd = s.num_heads, s.num_kv_heads, s.head_dim, self.value_dim
         n_store = 0 if self.shared_kv else nkv
-        width = (nh + n_store) * hd + n_store * vd
+        heads_width = (nh + n_store) * hd + n_store * vd
+        width = heads_width + (nh * vd if self.gate_name else 0)
         g = ctx.group(cache.group)
         tables = self.position.rotary_tables()
         qkv = linear(ctx, x, self.w_qkv, ctx.alloc((T, width)))
@@ -171,16 +187,32 @@ class PagedAttention(Part):
         ptr = lambda t: t.ptr if t is not None else None
         vfreq = ptr(self.value_freq)
         inter = 1 if getattr(s, "value_pairs_interleaved", False) else 0
-        k.zk_head_prep_ext(qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map, ptr(self.q_gain),
-                           ptr(self.k_gain), ptr(self.head_scale), float(s.norm_eps),
-                           tables[0].ptr if tables is not None else None, tables[1] if tables is not None else 0, vfreq,
-                           inter, cache.k.ptr, cache.v.ptr, T, nh, n_store, hd, vd, g.page_size,
-                           1 if cache.v_transposed else 0, ptr(self.in_bias), self.rot_scale,
-                           1 if self.rot_interleaved else 0, ctx.stream)
+        prep = (qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map, ptr(self.q_gain),
+                ptr(self.k_gain), ptr(self.head_scale), float(s.norm_eps),
+                tables[0].ptr if tables is not None else None, tables[1] if tables is not None else 0, vfreq,
+                inter, cache.k.ptr, cache.v.ptr, T, nh, n_store, hd, vd, g.page_size,
+                1 if cache.v_transposed else 0, ptr(self.in_bias), self.rot_scale,
+                1 if self.rot_interleaved else 0)
+        if self.unit_norm or width != heads_width:
+            k.zk_head_prep_unit(*prep, width, 1 if self.unit_norm else 0, ctx.stream)
+        else:
+            k.zk_head_prep_ext(*prep, ctx.stream)
         o = ctx.alloc((T, nh * vd))
         cap = float(s.softcap) if s.softcap else 0.0
         win = int(s.window) if s.window else 0
-        if cache.v_transposed and ctx.tuned and vd == hd:
+        masked = bool(self.chunk or self.unit_sink)
+        if masked and cache.v_transposed and ctx.tuned and vd == hd:
+            k.zk_attention_bf16_masked(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
+                                       ctx.q_start, ctx.ctx_len, o.ptr, ctx.R, ctx.n_multi, ctx.max_q_len,
+                                       ctx.max_ctx, nh, nkv, hd, g.page_size, s.scale, cap, win,
+                                       self.decode_chunk, ctx.workspace.ptr, ctx.workspace.nbytes, self.chunk,
+                                       1 if self.unit_sink else 0, ctx.stream)
+        elif masked:
+            k.zk_attention_plain_masked(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
+                                        ctx.req_of_token, ctx.positions, o.ptr, T, nh, nkv, hd, vd, g.page_size, s.scale,
+                                        cap, win, 1 if cache.v_transposed else 0, vfreq, inter, None, 0, self.chunk,
+                                        1 if self.unit_sink else 0, ctx.stream)
+        elif cache.v_transposed and ctx.tuned and vd == hd:
             k.zk_attention_bf16(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
                                 ctx.q_start, ctx.ctx_len, o.ptr, ctx.R, ctx.n_multi, ctx.max_q_len,
                                 ctx.max_ctx, nh, nkv, hd, g.page_size, s.scale, cap, win,
@@ -191,6 +223,9 @@ class PagedAttention(Part):
             k.zk_attention_plain_ext(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
                                      ctx.req_of_token, ctx.positions, o.ptr, T, nh, nkv, hd, vd, g.page_size, s.scale,
                                      cap, win, 1 if cache.v_transposed else 0, vfreq, inter, ctx.stream)
+        if self.gate_name:
+            # the heads times sigmoid(W_g x); the gate's columns lie behind the heads' in the product's rows
+            k.zk_gate_heads(o.ptr, qkv.ptr + heads_width * ITEMSIZE[ctx.dtype], width, T, nh * vd, ctx.stream)
         y = linear(ctx, o, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self if self.o_bias is None else None)
         if self.o_bias is not None:
             if getattr(ctx, "bias_welcome", None) is self:

@@ -43,12 +43,17 @@ class TensorReq:
 @dataclass(frozen=True)
 class PagedKV:
     """The mixer keeps keys and values per token, in pages.  ``window``: only the
-    last ``window`` positions are ever read again (None: all of them)."""
+    last ``window`` positions are ever read again (None: all of them).  ``chunk``: a query reads
+    the keys of its own chunk of ``chunk`` positions only (chunks counted from position 0), so
+    nothing before the chunk of the next token is ever read again.  ``state_bytes``: what the
+    mixer keeps per request beside its pages, whatever the request's length."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int]
     value_dim: Optional[int] = None     # size of a head's values where it differs from its keys'
     values_in_keys: bool = False        # a value is the first value_dim channels of its key: no value slab is kept
+    chunk: Optional[int] = None
+    state_bytes: int = 0
 
 
 @dataclass(frozen=True)

@@ -87,10 +87,11 @@ class Block(Part):
 
 
 class ParallelBlock(Part):
-    """x = norm(h); h += mixer(x) + ffn(x): one norm, both sublayers read it, and their results
-    are summed before they join the float stream (``ffn`` None: the mixer alone).  One kernel
-    does the sum, the mixer's output bias if it has one, the residual sum and the norm of
-    whatever runs next."""
+    """x = norm(h); h += mixer(x) + ffn(x): both sublayers read the same stream, and their results
+    are summed before they join it (``ffn`` None: the mixer alone).  With a second norm
+    ``pre_ffn`` the feed-forward reads that norm of the same h instead, and with
+    ``residual_scale`` m the sum joins as h += m (mixer + ffn).  One kernel does the sum, the
+    mixer's output bias if it has one, the residual sum and the norms of whatever runs next."""
     graph_safe = True      # its launches take what changes from step to step from device memory alone
 
     def __init__(self, spec):
@@ -100,36 +101,81 @@ class ParallelBlock(Part):
         self.norms = {"pre_mixer": build_part("norm", spec.norms["pre_mixer"])}
         self.mixer = build_part("mixer", spec.mixer)
         self.ffn = build_part("ffn", spec.ffn) if spec.ffn is not None else None
+        if self.ffn is not None and "pre_ffn" in spec.norms:
+            self.norms["pre_ffn"] = build_part("norm", spec.norms["pre_ffn"])
+        self.mult = float(getattr(spec, "residual_scale", 1.0))
 
     def children(self):
         return list(self.norms.values()) + [self.mixer] + ([self.ffn] if self.ffn is not None else [])
 
     def entry_norm(self):
+        """The norm of the stream that the block reads first, or both of them."""
+        if "pre_ffn" in self.norms:
+            return (self.norms["pre_mixer"], self.norms["pre_ffn"])
         return self.norms["pre_mixer"]
 
-    def forward(self, ctx, h: Tensor, cache, x_in: Tensor = None, next_norm=None, x_out: Tensor = None):
+    @staticmethod
+    def _fusable(norms) -> bool:
+        """Whether the closing kernel can make these norms: RMS norms of one eps and one kind of gain."""
+        return all(isinstance(n, RMSNorm) for n in norms) and \
+            len({(float(n.spec.eps), bool(n.spec.unit_offset)) for n in norms}) == 1
+
+    def _entry(self, ctx, h: Tensor, x_in):
+        """The block's own norms of the stream, from the caller where it brings them."""
+        mine = self.entry_norm()
+        if not isinstance(mine, tuple):
+            return (x_in if x_in is not None else mine.forward(ctx, h)), None
+        if isinstance(x_in, tuple):
+            return x_in
+        if not self._fusable(mine):
+            return mine[0].forward(ctx, h), mine[1].forward(ctx, h)
         T, H = h.shape
-        x = x_in if x_in is not None else self.norms["pre_mixer"].forward(ctx, h)
+        x1, x2 = ctx.alloc((T, H)), ctx.alloc((T, H))
+        sp = mine[0].spec
+        ctx.k.zk_sum_norm_pair(h.ptr, None, 0, None, 0, None, 1.0, mine[0].weight.ptr, x1.ptr, mine[1].weight.ptr, x2.ptr,
+                               float(sp.eps), int(sp.unit_offset), T, H, ctx.stream)
+        return x1, x2
+
+    def forward(self, ctx, h: Tensor, cache, x_in=None, next_norm=None, x_out=None):
+        """``x_in``, ``next_norm`` and ``x_out`` are single or pairs, as ``entry_norm`` of this block
+        and of the next one are."""
+        T, H = h.shape
+        x, x2 = self._entry(ctx, h, x_in)
         # the mixer's result has to outlive the feed-forward's products: no partial sums in the
-        # products' shared workspace; its output bias is added by the joining kernel
-        ctx.sums_welcome, ctx.bias_welcome, ctx.result_bias = None, self.mixer, None
+        # products' shared workspace (a float plane in the step's own memory is welcome); its
+        # output bias is added by the joining kernel
+        ctx.sums_welcome, ctx.bias_welcome, ctx.result_bias, ctx.plane_welcome = None, self.mixer, None, self.mixer
         a = self.mixer.forward(ctx, x, cache)
-        bias, ctx.bias_welcome, ctx.result_bias = ctx.result_bias, None, None
+        bias, ctx.bias_welcome, ctx.result_bias, ctx.plane_welcome = ctx.result_bias, None, None, None
         m = None
         if self.ffn is not None:
             ctx.sums_welcome = self.ffn
-            m = self.ffn.forward(ctx, x)
+            m = self.ffn.forward(ctx, x2 if x2 is not None else x)
             ctx.sums_welcome = None
-        ns = next_norm.spec if isinstance(next_norm, RMSNorm) else None
-        out = None
-        if ns is not None:
-            out = ctx.alloc((T, H)) if x_out is None else Tensor(x_out.ptr, (T, H), ctx.dtype, x_out.owner)
+        nxt = next_norm if isinstance(next_norm, tuple) else ((next_norm,) if next_norm is not None else ())
+        if not nxt or not self._fusable(nxt) or len(nxt) > 2:
+            nxt = ()             # norms the closing kernel does not know: the next block applies them
+        outs = []
+        for i in range(len(nxt)):
+            buf = (x_out[i] if isinstance(x_out, (tuple, list)) else x_out if i == 0 else None) if x_out is not None else None
+            outs.append(ctx.alloc((T, H)) if buf is None else Tensor(buf.ptr, (T, H), ctx.dtype, buf.owner))
         planes = lambda t: t.shape[0] if (t is not None and t.layout == "parts") else 0
-        ctx.k.zk_sum_norm(h.ptr, a.ptr, planes(a), m.ptr if m is not None else None, planes(m),
-                          bias.ptr if bias is not None else None, next_norm.weight.ptr if ns is not None else None,
-                          float(ns.eps) if ns is not None else 0.0, int(ns.unit_offset) if ns is not None else 0,
-                          out.ptr if out is not None else None, T, H, ctx.stream)
-        return out
+        ptr = lambda t: t.ptr if t is not None else None
+        if self.mult == 1.0 and len(nxt) <= 1:
+            ns = nxt[0].spec if nxt else None
+            ctx.k.zk_sum_norm(h.ptr, a.ptr, planes(a), ptr(m), planes(m), ptr(bias), nxt[0].weight.ptr if nxt else None,
+                              float(ns.eps) if ns is not None else 0.0, int(ns.unit_offset) if ns is not None else 0,
+                              outs[0].ptr if outs else None, T, H, ctx.stream)
+        else:
+            ns = nxt[0].spec if nxt else None
+            w = [n.weight.ptr for n in nxt] + [None, None]
+            o = [t.ptr for t in outs] + [None, None]
+            ctx.k.zk_sum_norm_pair(h.ptr, a.ptr, planes(a), ptr(m), planes(m), ptr(bias), self.mult, w[0], o[0], w[1], o[1],
+                                   float(ns.eps) if ns is not None else 0.0, int(ns.unit_offset) if ns is not None else 0,
+                                   T, H, ctx.stream)
+        if not outs:
+            return None
+        return tuple(outs) if isinstance(next_norm, tuple) else outs[0]
 
 
 def _block(spec):

@@ -70,6 +70,43 @@ class GatedMLP(Part):
         return linear(ctx, a, self.w_down, ctx.alloc((T, s.hidden_size)), last_of=self)
 
 
+UNARY_CODES = {"relu2": 0}     # max(z, 0)^2
+
+
+class MLP(Part):
+    """act(x Wu^T) Wd^T without a gate; the activation rides in the first product's epilogue where
+    the matrix-core product serves the step."""
+    graph_safe = True      # its launches take what changes from step to step from device memory alone
+
+    def __init__(self, spec):
+        if spec.activation not in UNARY_CODES:
+            raise ValueError(f"activation must be one of {sorted(UNARY_CODES)}, got {spec.activation!r}")
+        self.spec = spec
+        self.w_up = self.w_down = None
+
+    def tensor_reqs(self) -> List[TensorReq]:
+        s = self.spec
+        return [TensorReq(s.names["up"], (s.intermediate_size, s.hidden_size)),
+                TensorReq(s.names["down"], (s.hidden_size, s.intermediate_size))]
+
+    def load(self, weights, rt, dtype):
+        s = self.spec
+        strip = getattr(weights, "wants_strip", None)
+        self.w_up = weights.matrix([s.names["up"]], strip=bool(strip and strip(s.hidden_size)))
+        self.w_down = weights.matrix([s.names["down"]], strip=bool(strip and strip(s.intermediate_size)))
+
+    def forward(self, ctx, x: Tensor) -> Tensor:
+        s = self.spec
+        T, I = x.shape[0], s.intermediate_size
+        if tuned_gemm(ctx, s.hidden_size) and ctx.k.has("zk_gemm_bf16_unary"):
+            a = linear(ctx, x, self.w_up, ctx.alloc((T, I)), epilogue=s.activation)
+        else:
+            up = linear(ctx, x, self.w_up, ctx.alloc((T, I)))
+            a = ctx.alloc((T, I))
+            ctx.k.zk_unary_act(up.ptr, a.ptr, T * I, UNARY_CODES[s.activation], ctx.stream)
+        return linear(ctx, a, self.w_down, ctx.alloc((T, s.hidden_size)), last_of=self)
+
+
 class RoutedMLP(Part):
     """A mixture of small gated layers: sigmoid scores from a float router product, the ``top_k``
     largest chosen on the device (the lower index among equals), the chosen scores as weights on
@@ -154,4 +191,5 @@ class RoutedMLP(Part):
 
 
 register_part("ffn", "gated_mlp", GatedMLP)
+register_part("ffn", "mlp", MLP)
 register_part("ffn", "routed_mlp", RoutedMLP)

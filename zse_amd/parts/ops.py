@@ -6,7 +6,7 @@ import ctypes
 from ..runtime.device import BF16, F32, Tensor
 
 
-EPILOGUES = {None: 0, "softcap": 1, "gelu_tanh": 2, "silu": 3, "relu": 5, "clamped_swiglu": 6}
+EPILOGUES = {None: 0, "softcap": 1, "gelu_tanh": 2, "silu": 3, "relu": 5, "clamped_swiglu": 6, "relu2": 7}
 GATED = ("gelu_tanh", "silu", "relu", "clamped_swiglu")
 
 
@@ -17,7 +17,7 @@ def tuned_gemm(ctx, K: int) -> bool:
 
 
 def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0.0, last_of=None,
-           sums_ok: bool = False) -> Tensor:
+           sums_ok: bool = False, lda: int = 0) -> Tensor:
     """out[M, N] = x[M, K] @ w[N, K]^T with float accumulation.
 
     ``out`` may be float32 (logits) or the activation type.  In the 32-bit
@@ -26,6 +26,9 @@ def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0
     "softcap" applies cap * tanh(x / cap); "gelu_tanh" / "silu" / "relu" take w as
     [2N, K], gate rows first, and store act(gate) * up; "clamped_swiglu" likewise, with ``cap`` as
     its limit: g = min(gate, cap), u = clamp(up, -cap, cap), g sigmoid(1.702 g) (u + 1).
+
+    "relu2" stores max(x, 0)^2.  ``lda``: the distance between the rows of ``x`` in elements
+    where they are the first K columns of wider rows (0: K).
 
     ``last_of``: the part whose result this product is (it passes itself).  When the block
     that called that very part has said that partial sums are welcome (``ctx.sums_welcome`` is
@@ -52,18 +55,23 @@ def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0
     out_f32 = 1 if out.dtype == F32 else 0
     k = ctx.k
     strip = w.layout == "strip"
-    if strip and not tuned_gemm(ctx, K):
-        raise ValueError("linear: weights in strip layout need the matrix-core product")
-    if tuned_gemm(ctx, K):
+    lda = int(lda) or K
+    if lda < K:
+        raise ValueError(f"linear: rows {lda} apart hold no {K} columns")
+    # the matrix-core product reads whole 16-byte pieces: rows that begin at such addresses
+    tuned = tuned_gemm(ctx, K) and lda % 8 == 0 and x.ptr % 16 == 0
+    if (strip or epilogue is not None) and not tuned:
+        raise ValueError("linear: weights in strip layout and epilogues need the matrix-core product")
+    if tuned:
         ws = getattr(ctx, "gemm_workspace", None)      # lets a product of few columns split K over blocks
         welcome = sums_ok or (last_of is not None and getattr(ctx, "sums_welcome", None) is last_of)
         parts = ctypes.c_int(0) if (welcome and ws is not None) else None
-        k.zk_gemm_bf16(x.ptr, K, w.ptr, out.ptr, N, out_f32, M, N, K, EPILOGUES[epilogue], float(cap),
+        k.zk_gemm_bf16(x.ptr, lda, w.ptr, out.ptr, N, out_f32, M, N, K, EPILOGUES[epilogue], float(cap),
                        1 if strip else 0, ws.ptr if ws is not None else None,
                        ws.nbytes if ws is not None else 0, ctypes.byref(parts) if parts is not None else None,
                        ctx.stream)
         if parts is not None and parts.value > 0:
             return Tensor(ws.ptr, (parts.value, M, N), F32, ws.owner, layout="parts")
     else:
-        k.zk_gemm_plain(x.ptr, K, w.ptr, out.ptr, N, out_f32, M, N, K, ctx.stream)
+        k.zk_gemm_plain(x.ptr, lda, w.ptr, out.ptr, N, out_f32, M, N, K, ctx.stream)
     return out

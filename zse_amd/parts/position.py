@@ -21,6 +21,8 @@ class Rotary(Part):
     def __init__(self, spec):
         if spec.rotary_dim % 2 or not (0 < spec.rotary_dim <= spec.head_dim):
             raise ValueError(f"rotary_dim must be even and in (0, head_dim], got {spec.rotary_dim}")
+        if getattr(spec, "linear_factor", None) is not None and not spec.linear_factor > 0:
+            raise ValueError(f"linear_factor must be positive, got {spec.linear_factor}")
         self.spec = spec
         self.inv_freq = None
 
@@ -38,6 +40,9 @@ class Rotary(Part):
             hi = min(math.ceil(at(slow)), s.rotary_dim - 1)
             ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
             f = f / factor * ramp + f * (1.0 - ramp)
+        linear = getattr(s, "linear_factor", None)
+        if linear is not None:
+            f = f / float(linear)
         return f.astype(np.float32)
 
     def magnitude(self) -> float:

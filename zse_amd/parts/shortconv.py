@@ -1,6 +1,7 @@
 """A short causal convolution over time on each channel, added to its input:
 out_t = x_t + sum_j w[:, j] x_(t - taps + 1 + j), rows before a sequence's start being zero
-(``residual`` False: the sum alone; ``activation`` "silu": silu of the result).
+(``residual`` False: the sum alone; ``activation`` "silu": silu of the result; ``bias``: a
+number per channel that the sum starts from).
 The ``taps - 1`` rows before a request's next token are its state (float, in its state slot,
 which starts as zeros): a step reads them for its first tokens and renews them afterwards.
 """
@@ -21,20 +22,23 @@ class ShortConv(Part):
         if getattr(spec, "activation", None) not in (None, "silu"):
             raise ValueError(f"a convolution's activation is None or 'silu', got {spec.activation!r}")
         self.spec = spec
-        self.weight = None
+        self.weight = self.bias = None
+        self.bias_name = getattr(spec, "bias", None)
         self.names = [spec.weight] if isinstance(spec.weight, str) else list(spec.weight)
 
     def tensor_reqs(self) -> List[TensorReq]:
         s = self.spec
+        extra = [TensorReq(self.bias_name, (s.size,), ROLE_GAIN)] if self.bias_name else []
         if len(self.names) == 1:
-            return [TensorReq(self.names[0], (s.size, s.taps), ROLE_GAIN)]
+            return [TensorReq(self.names[0], (s.size, s.taps), ROLE_GAIN)] + extra
         sizes = getattr(s, "channel_counts", None)
         if sizes is None or len(sizes) != len(self.names) or sum(sizes) != s.size:
             raise ValueError("a convolution over several tensors says how many channels each has (channel_counts)")
-        return [TensorReq(n, (c, s.taps), ROLE_GAIN) for n, c in zip(self.names, sizes)]
+        return [TensorReq(n, (c, s.taps), ROLE_GAIN) for n, c in zip(self.names, sizes)] + extra
 
     def load(self, weights, rt, dtype):
         self.weight = weights.vectors(self.names)
+        self.bias = weights.vector(self.bias_name) if self.bias_name else None
 
     def state_bytes(self) -> int:
         return (self.spec.taps - 1) * self.spec.size * 4
@@ -52,14 +56,16 @@ class ShortConv(Part):
         words = ctx.state.shape[1] if ctx.state is not None else 0
         residual = 1 if getattr(s, "residual", True) else 0
         act = 1 if getattr(s, "activation", None) == "silu" else 0
+        bias = self.bias.ptr if self.bias is not None else None
         if ctx.max_q_len == 1 and T == ctx.R:
             # every request brings one token: one launch computes and moves the state on
-            k.zk_short_conv_token_ext(x.ptr, ld, self.weight.ptr, state, words, state_offset // 4, ctx.positions,
-                                      ctx.req_of_token, ctx.q_start, ctx.slot_of_req, out.ptr, s.size, T, s.size, s.taps,
-                                      residual, act, ctx.stream)
+            k.zk_short_conv_token_bias(x.ptr, ld, self.weight.ptr, state, words, state_offset // 4, ctx.positions,
+                                       ctx.req_of_token, ctx.q_start, ctx.slot_of_req, out.ptr, s.size, T, s.size, s.taps,
+                                       residual, act, bias, ctx.stream)
             return out
-        k.zk_short_conv_ext(x.ptr, ld, self.weight.ptr, state, words, state_offset // 4, ctx.positions, ctx.req_of_token,
-                            ctx.q_start, ctx.slot_of_req, out.ptr, s.size, T, s.size, s.taps, residual, act, ctx.stream)
+        k.zk_short_conv_bias(x.ptr, ld, self.weight.ptr, state, words, state_offset // 4, ctx.positions, ctx.req_of_token,
+                             ctx.q_start, ctx.slot_of_req, out.ptr, s.size, T, s.size, s.taps, residual, act, bias,
+                             ctx.stream)
         k.zk_short_conv_state_ext(x.ptr, ld, state, words, state_offset // 4, ctx.q_start, ctx.slot_of_req, ctx.R, s.size,
                                   s.taps, ctx.stream)
         return out

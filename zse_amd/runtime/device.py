@@ -193,6 +193,20 @@ KERNEL_SIGNATURES = {
     "zk_sum_norm": [_VP, _VP, _I, _VP, _I, _VP, _VP, _F, _I, _VP, _I, _I, _VP],
     "zk_add_bias": [_VP, _VP, _I, _I, _VP],
     "zk_planes_sum": [_VP, _I, _VP, _I, _I, _VP],
+    "zk_sum_norm_pair": [_VP, _VP, _I, _VP, _I, _VP, _F, _VP, _VP, _VP, _VP, _F, _I, _I, _I, _VP],
+    "zk_weighted_sum": [_VP, _F, _VP, _F, _VP, _F, _VP, _F, _VP, _I, _I, _VP],
+    "zk_attention_plain_masked": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _F,
+                                  _I, _I, _VP, _I, _VP, _I, _I, _I, _VP],
+    "zk_head_prep_unit": [_VP, _VP, _VP, _VP, _VP, _VP, _F, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I,
+                          _VP, _F, _I, _I, _I, _VP],
+    "zk_short_conv_bias": [_VP, _I, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP],
+    "zk_short_conv_token_bias": [_VP, _I, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP],
+    "zk_unary_act": [_VP, _VP, _SZ, _I, _VP],
+    "zk_gate_heads": [_VP, _VP, _I, _I, _I, _VP],
+    "zk_gla": [_VP, _I, _I, _I, _VP, _I, _VP, _I, _VP, _F, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I,
+               _F, _VP],
+    "zk_selective_scan": [_VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I,
+                          _I, _VP],
 }
 # present only in the bf16 library
 BF16_KERNEL_SIGNATURES = {

@@ -82,8 +82,10 @@ def check_entries(entries: Dict[str, st.TensorEntry], reqs: Iterable[TensorReq],
     skip = {_strip(n, prefixes) for n in ignored}
     missing = [want[k].name for k in want if k not in have]
     unexpected = [have[k].name for k in have if k not in want and k not in skip]
+    # an extent of -1 in a request is one that the checkpoint itself says (the part reads it at load)
+    fits = lambda got, asked: len(got) == len(asked) and all(a == -1 or a == g for g, a in zip(got, asked))
     wrong_shape = [(have[k].name, have[k].shape, want[k].shape) for k in want
-                   if k in have and tuple(have[k].shape) != tuple(want[k].shape)]
+                   if k in have and not fits(tuple(have[k].shape), tuple(want[k].shape))]
     wrong_dtype = [(have[k].name, have[k].dtype) for k in want
                    if k in have and have[k].dtype not in SRC_TAGS]
     if missing or unexpected or wrong_shape or wrong_dtype:
@@ -142,6 +144,14 @@ class _Source:
             self.bytes_on_device += out.nbytes
             self._cache[key] = out
         return self._cache[key]
+
+    def shape_of(self, name: str) -> Tuple[int, ...]:
+        """The tensor's shape in the source; a part that left an extent open (-1) reads it here."""
+        shape = tuple(int(v) for v in self._shape(name))
+        if any(v < 0 for v in shape):
+            raise ValueError(f"tensor {name}: this source holds no tensors of its own, so every extent must be "
+                             f"given; asked for {shape}")
+        return shape
 
     def vector(self, name: str) -> Tensor:
         key = ("v", _strip(name, self.prefixes))
