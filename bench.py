@@ -473,6 +473,25 @@ def pubunex_config(width, heads, kv_heads, dim, ff, groups, vocab, window):
     return {"architecture": "Pubunex", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": layers}
 
 
+def bumolix_config(width, heads, kv_heads, dim, ff, groups, vocab, window):
+    """``groups`` times (parallel, parallel, selective scan), each with a squared-relu feed-forward.
+    A parallel mixer is a chunked attention with the relative's heads beside a gated linear
+    attention with half as many heads of dim / 2 keys and dim values (the relative's mLSTM has
+    heads of that shape); the scan has 2 width channels of 16 state values."""
+    par = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": 8.0 / dim,
+                    "mask": {"size": window}, "rot": {"base": 10000.0, "dims": dim // 2, "scaling": {"factor": 2.0}}},
+           "right": {"heads": max(heads // 2, 1), "dim": dim // 2, "vdim": dim, "tau": 16.0, "rank": 16},
+           "left_scale": 1.0, "right_scale": 1.0}
+    scan = {"inner": 2 * width, "state": 16, "dt_rank": width // 16, "conv": 4}
+    layers = []
+    for _ in range(groups):
+        layers += [{"type": "parallel", "mixer": dict(par), "mlp": {"kind": "dense", "ff": ff}},
+                   {"type": "parallel", "mixer": dict(par), "mlp": {"kind": "dense", "ff": ff}},
+                   {"type": "mamba1", "mixer": dict(scan), "mlp": {"kind": "dense", "ff": ff}}]
+    return {"architecture": "Bumolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+            "layers": layers}
+
+
 # what is timed, beside which relative, against which plain implementation it is checked first, and
 # the deviations of the random tensors that are not drawn like matrices or gains
 DESIGNS = {
@@ -481,6 +500,9 @@ DESIGNS = {
     "pubunex": dict(name="Pubunex", make=pubunex_config, plain="pubunex_plain",
                     std_of={".conv": 0.3, "A_log": 0.5, "dt_bias": 0.5, "mix.norm": 1.0, "dkv.norm": 1.0, ".sink": 1.0, ".b": 0.02,
                             "router": 0.1},
+                    beside=("dafotar", "Dafotar", dafotar_config)),
+    "bumolix": dict(name="Bumolix", make=bumolix_config, plain="bumolix_plain",
+                    std_of={".b": 0.02, ".conv": 0.3, "A_log": 0.5, "dt.b": 0.5, "a2.b": 1.0, ".D": 0.5, "norm": 0.5},
                     beside=("dafotar", "Dafotar", dafotar_config)),
 }
 
@@ -615,9 +637,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--design", choices=sorted(DESIGNS), default=None,
                     help="instead of the default workload: prefill and decode of this design beside its closest relative "
-                         "(Dafotar beside Gemma 2, Pubunex beside Dafotar) at equal layer sizes")
+                         "(Dafotar beside Gemma 2, Pubunex and Bumolix beside Dafotar) at equal layer sizes")
     ap.add_argument("--design-sizes", default="w1024,w2048,w4096", help="with --design: which of " + ", ".join(DESIGN_SIZES))
-    ap.add_argument("--only-model", choices=["dafotar", "gemma2", "pubunex"], default=None, help="with --design, a profiling aid: one of the two")
+    ap.add_argument("--only-model", choices=["bumolix", "dafotar", "gemma2", "pubunex"], default=None, help="with --design, a profiling aid: one of the two")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)

@@ -102,6 +102,8 @@ class AttentionSpec:
     unit_sink: bool = False                  # a sink of score 0 without a value: weights exp(s_j) / (1 + sum exp(s))
     qk_unit_norm: bool = False               # q and k divided by their root mean square per head, no gain, AFTER rotation
     gate: Optional[str] = None               # [num_heads * value_dim, hidden]: heads times sigmoid(W_g x) before W_o
+    wide_weights: bool = False               # the softmax's weights are not rounded to 8 bits of mantissa before they
+    #                                          meet the values (the matrix-core kernel sends them in two halves)
 
 
 @dataclass(frozen=True)

@@ -34,6 +34,7 @@
 // a single query token fills only g of a tile's columns, and the narrower tile
 // halves both the accumulator registers and the wasted work, so two waves fit a SIMD.
 #include "common.h"
+#include "packed_call.h"
 
 #include <algorithm>
 
@@ -72,7 +73,23 @@ struct AttnParams {
   int nchunks;            // split: chunks the grid covers
   int from_window;        // decode: block 0 of a request is the one its window begins in
   int chunk;              // decoded tokens on 16-wide tiles: keys a wave takes, 32 or 64
+  int mask_chunk;         // > 0: a row sees the keys of its own chunk of this many positions only (no window then)
+  int sink;               // 1: a key of score 0 without a value joins every row's denominator
+  int wide_weights;       // 1: a weight meets the values as two bf16 numbers, its rounded value and what the
+                          // rounding left (16 bits of mantissa instead of 8; one more product a tile)
 };
+
+// The first key a row at position ``pos`` sees.  It never decreases as pos grows, which is all
+// the kernels' bounds over groups and blocks of rows rest on.
+__device__ __forceinline__ int first_key(const AttnParams& p, int pos) {
+  if (p.mask_chunk > 0) return pos - pos % p.mask_chunk;
+  return p.window > 0 ? max(0, pos - p.window + 1) : 0;
+}
+
+// What the sink adds to a row's sum of weights: 2^(0 - m), scores and maximum in the log2 domain.
+__device__ __forceinline__ float sink_weight(const AttnParams& p, float m) {
+  return p.sink ? __builtin_amdgcn_exp2f(-m) : 0.f;
+}
 
 __device__ __forceinline__ float score_log2(const AttnParams& p, float dot) {
   if (p.softcap > 0.f) {
@@ -134,7 +151,7 @@ __global__ __launch_bounds__(256, (HD16 <= 8 && !PAIR) ? 2 : 1) void attn_mfma_k
     if (ga != gb) {
       auto tiles_of = [&](int gr) {
         const int lo = start + gr * p.tpw, hi = start + min(n, (gr + 1) * p.tpw) - 1;
-        const int klo = p.window > 0 ? max(0, lo - p.window + 1) : 0;
+        const int klo = first_key(p, lo);
         return hi / 32 - klo / 32 + 1;
       };
       const int ta = tiles_of(ga), tb = tiles_of(gb);
@@ -157,14 +174,14 @@ __global__ __launch_bounds__(256, (HD16 <= 8 && !PAIR) ? 2 : 1) void attn_mfma_k
   const int pos = start + t0 + (row_ok ? tok : 0);
   const int head = kvh * g + (row_ok ? hq : 0);
   const int pos_lo = start + t0, pos_hi = start + t0 + ntok - 1;
-  int key_lo = p.window > 0 ? max(0, pos_lo - p.window + 1) : 0;
+  int key_lo = first_key(p, pos_lo);
   int key_hi = pos_hi;
   if (SPLIT) {
     key_lo = max(key_lo, chunk * ATT_CHUNK);
     key_hi = min(key_hi, chunk * ATT_CHUNK + ATT_CHUNK - 1);
   }
   if (SPLIT && key_lo > key_hi) return;
-  const int row_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int row_lo = first_key(p, pos);
   const int* table = p.block_table + (size_t)r * p.max_blocks;
   const int hd = p.hd, bsh = p.bs_shift, bmask = p.bs - 1, nkv = p.nkv;
 
@@ -194,7 +211,7 @@ __global__ __launch_bounds__(256, (HD16 <= 8 && !PAIR) ? 2 : 1) void attn_mfma_k
   // last row's window; no range at all unless every lane holds a row): tiles inside this range
   // need no mask
   const int all_hi = ntok * g == 32 ? pos_lo : -1;
-  const int all_lo = p.window > 0 ? max(0, pos_hi - p.window + 1) : 0;
+  const int all_lo = first_key(p, pos_hi);
 
   // The pages of a tile are looked up a tile ahead as well, so that no load waits for a table
   // entry: the lane's key row, and the four places its V pieces come from.
@@ -307,6 +324,17 @@ __global__ __launch_bounds__(256, (HD16 <= 8 && !PAIR) ? 2 : 1) void attn_mfma_k
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][0], pb[0], o[dt], 0, 0, 0);
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][1], pb[1], o[dt], 0, 0, 0);
     }
+    if (p.wide_weights) {
+#pragma unroll
+      for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) pb[h][e] = (__bf16)(s[8 * h + e] - (float)pb[h][e]);
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++) {
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][0], pb[0], o[dt], 0, 0, 0);
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][1], pb[1], o[dt], 0, 0, 0);
+      }
+    }
   
   };
   {
@@ -377,7 +405,7 @@ __global__ __launch_bounds__(256, (HD16 <= 8 && !PAIR) ? 2 : 1) void attn_mfma_k
       __syncthreads();
     }
     if (phase != 0 || !row_ok) return;
-    const float inv = 1.f / l_all;
+    const float inv = 1.f / (l_all + sink_weight(p, m_all));
     __bf16* orow = p.out + ((size_t)trow * p.nh + head) * hd;
 #pragma unroll
     for (int dt = 0; dt < DT; dt++)
@@ -440,7 +468,7 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
   const int g = p.nh / p.nkv;
   // the block's keys: from the window of its first row to its last row
   const int blk_lo = start + bi * per_block, blk_hi = start + min(n, (bi + 1) * per_block) - 1;
-  int key_lo = p.window > 0 ? max(0, blk_lo - p.window + 1) : 0;
+  int key_lo = first_key(p, blk_lo);
   int key_hi = blk_hi;
   if (SPLIT) {
     const int first_tile = key_lo / 32 + range * p.chunk;
@@ -457,9 +485,9 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
   const int pos = start + (row_ok ? t0 + tok : 0);
   const int head = kvh * g + (row_ok ? hq : 0);
   const int pos_lo = start + t0, pos_hi = start + t0 + ntok - 1;          // ntok == 0: no keys at all
-  const int row_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int row_lo = first_key(p, pos);
   const int all_hi = ntok * g == 32 ? pos_lo : -1;
-  const int all_lo = p.window > 0 ? max(0, pos_hi - p.window + 1) : 0;
+  const int all_lo = first_key(p, pos_hi);
   const int* table = p.block_table + (size_t)r * p.max_blocks;
   const int bsh = p.bs_shift, bmask = p.bs - 1, nkv = p.nkv;
 
@@ -630,6 +658,18 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)vr, pb[0], o[dt], 0, 0, 0);
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(vr + 16), pb[1], o[dt], 0, 0, 0);
     }
+    if (p.wide_weights) {
+#pragma unroll
+      for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) pb[h][e] = (__bf16)(s[8 * h + e] - (float)pb[h][e]);
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++) {
+        const __bf16* vr = vb + min(dt * 32 + lr, HD - 1) * VLD;
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)vr, pb[0], o[dt], 0, 0, 0);
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(vr + 16), pb[1], o[dt], 0, 0, 0);
+      }
+    }
   };
 
   // Every wave takes every tile of the block, also the few near the diagonal (or before its
@@ -670,7 +710,7 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
         po[(dt * 4 + j) * 64] = f32x4{o[dt][4 * j], o[dt][4 * j + 1], o[dt][4 * j + 2], o[dt][4 * j + 3]};
     return;
   }
-  const float inv = 1.f / l_run;
+  const float inv = 1.f / (l_run + sink_weight(p, m_run));
   __bf16* orow = p.out + ((size_t)trow * p.nh + head) * HD;
 #pragma unroll
   for (int dt = 0; dt < DT; dt++)
@@ -707,7 +747,7 @@ __global__ __launch_bounds__(64) void attn_portion_join_kernel(AttnParams p, int
   const int tok = lr / g, hq = lr - tok * g;
   if (tok >= ntok) return;
   const int blk_lo = start + bi * per_block, blk_hi = start + min(n, (bi + 1) * per_block) - 1;
-  const int key_lo = p.window > 0 ? max(0, blk_lo - p.window + 1) : 0;
+  const int key_lo = first_key(p, blk_lo);
   const int ranges = (blk_hi / 32 - key_lo / 32) / p.chunk + 1;
   const size_t slot0 = ((((size_t)blockIdx.z * p.nkv + kvh) * row_blocks + rows_x) * p.nchunks) * 4 + wave;
   float m = -INFINITY;
@@ -725,7 +765,7 @@ __global__ __launch_bounds__(64) void attn_portion_join_kernel(AttnParams p, int
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[j] += w * po[j * 64];
   }
-  const float inv = 1.f / l;
+  const float inv = 1.f / (l + sink_weight(p, m));
   __bf16* orow = p.out + ((size_t)(qs + t0 + tok) * p.nh + kvh * g + hq) * p.hd;
 #pragma unroll
   for (int j = 0; j < 4; j++) {
@@ -753,7 +793,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   // Where the window is much shorter than the longest context, the grid covers a window's
   // blocks only and counts them from the block the request's window begins in.
   int block_x = blockIdx.x;
-  if (p.from_window) block_x += max(0, p.ctx_len[r] - p.window) / (4 * p.chunk);
+  if (p.from_window) block_x += first_key(p, max(p.ctx_len[r] - 1, 0)) / (4 * p.chunk);
   const int chunk = block_x * 4 + wave;
   const int* table = p.block_table + (size_t)r * p.max_blocks;
   const int hd = p.hd, bsh = p.bs_shift, bmask = p.bs - 1, nkv = p.nkv;
@@ -775,7 +815,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const int n = p.q_start[r + 1] - p.q_start[r];
   if (n <= 0) return;
   const int pos = p.ctx_len[r] - 1;
-  const int row_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int row_lo = first_key(p, pos);
   // a block whose four chunks all lie past the context or before the window ends here, all
   // its waves alike: the grid is sized for the longest context the caller allows
   const int first_chunk = block_x * 4;
@@ -870,6 +910,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
         const float pe = __builtin_amdgcn_exp2f(s[t][i] - m_use);
         rs += pe;
         pb8[4 * t + i] = (__bf16)pe;
+        s[t][i] = pe;
       }
     rs += __shfl_xor(rs, 16, 64);
     rs += __shfl_xor(rs, 32, 64);
@@ -879,6 +920,14 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     for (int dt = 0; dt < DT; dt++) {
       o[dt] *= corr;
       o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb8, o[dt], 0, 0, 0);
+    }
+    if (p.wide_weights) {
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) pb8[4 * t + i] = (__bf16)(s[t][i] - (float)pb8[4 * t + i]);
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++) o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb8, o[dt], 0, 0, 0);
     }
   }
   // the block's four chunks are joined here, in chunk order: one partial result per 256 keys
@@ -927,7 +976,8 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
                                                            const int* __restrict__ q_start,
                                                            const int* __restrict__ ctx_len,
                                                            __bf16* __restrict__ out, int nh, int hd,
-                                                           int window, int r_begin, int nchunks, int span) {
+                                                           int window, int r_begin, int nchunks, int span,
+                                                           int mask_chunk, int sink) {
   __shared__ float wgt[ATT_MAX_CHUNKS];
   __shared__ float red[17];
   const int rr = blockIdx.x, head = blockIdx.y;
@@ -935,7 +985,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
   const int n = q_start[r + 1] - q_start[r];
   if (n <= 0) return;
   const int pos = ctx_len[r] - 1;
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = mask_chunk > 0 ? pos - pos % mask_chunk : window > 0 ? max(0, pos - window + 1) : 0;
   const int c0 = lo / span, c1 = pos / span;
   const size_t base = ((size_t)rr * nh + head) * nchunks;
   const int np = c1 - c0 + 1;
@@ -963,7 +1013,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
     l += part_ml[(base + c) * 2 + 1] * w;
   }
   l = block_sum(l, red);
-  const float inv = 1.f / l;
+  const float inv = 1.f / (l + (sink ? __builtin_amdgcn_exp2f(-m) : 0.f));
   __bf16* orow = out + ((size_t)q_start[r] * nh + head) * hd;
   for (int d = threadIdx.x; d < hd; d += 256) {
     const float* po = part_o + (base + c0) * hd + d;
@@ -1047,12 +1097,12 @@ static size_t portion_split_bytes(long row_blocks, int nkv, int hd, int ranges) 
 // results).  No split unless it at least halves the longest block's tiles; at most
 // ATT_MOST_RANGES ranges for the longest block of rows the caller's limits allow (bound_tiles),
 // which bounds the workspace.
-static int portion_ranges(int max_q_len, int max_ctx, int window, int per_block, int nkv, int r_prefill,
+static int portion_ranges(int max_q_len, int max_ctx, int window, int mask_chunk, int per_block, int nkv, int r_prefill,
                           int bound_tiles) {
   const int row_blocks = (max_q_len + per_block - 1) / per_block;
   auto tiles_of = [&](int bi) {
     const int lo = max_ctx - max_q_len + bi * per_block, hi = std::min(max_ctx, lo + per_block) - 1;
-    const int klo = window > 0 ? std::max(0, lo - window + 1) : 0;
+    const int klo = mask_chunk > 0 ? lo - lo % mask_chunk : window > 0 ? std::max(0, lo - window + 1) : 0;
     return hi / 32 - klo / 32 + 1;
   };
   int longest = 0;
@@ -1127,11 +1177,16 @@ long long zk_attention_bf16_max_context(int nh, int nkv, int hd, int decode_chun
 // a request's result not to depend on the rest of the batch passes the same value in every
 // step.  32 gives twice the waves, each with one load from memory in its chain instead of
 // two: better for few requests with short contexts, worse for many.
-int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const void* vcache_t,
-                      const int* block_table, int max_blocks, const int* q_start, const int* ctx_len,
-                      void* out, int R, int r_prefill, int max_q_len, int max_ctx, int nh, int nkv,
-                      int hd, int bs, float scale, float softcap, int window, int decode_chunk,
-                      void* workspace, size_t workspace_bytes, void* stream) {
+// mask_chunk > 0: a row sees the keys of its own chunk of that many positions (counted from
+// position 0) instead of a window; sink: a key of score 0 without a value in every denominator;
+// wide_weights: the weights keep 16 bits of mantissa in the product with the values.
+int zk_attention_bf16_masked(const void* q, int q_stride, const void* kcache, const void* vcache_t,
+                             const int* block_table, int max_blocks, const int* q_start, const int* ctx_len,
+                             void* out, int R, int r_prefill, int max_q_len, int max_ctx, int nh, int nkv,
+                             int hd, int bs, float scale, float softcap, int window, int decode_chunk,
+                             void* workspace, size_t workspace_bytes, int mask_chunk, int sink, int wide_weights,
+                             void* stream) {
+  ZK_REQUIRE(mask_chunk >= 0 && (mask_chunk == 0 || window == 0), "zk_attention_bf16: a window or a chunk, not both");
   ZK_REQUIRE(R >= 0 && r_prefill >= 0 && r_prefill <= R, "zk_attention_bf16: bad request counts");
   ZK_REQUIRE(zk_attention_bf16_supports(nh, nkv, hd, bs), "zk_attention_bf16: sizes not supported "
              "(head_dim 16/32/64/128/256, at most 32 heads a KV head, page size a power of two from 4)");
@@ -1159,6 +1214,7 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
   p.nh = nh; p.nkv = nkv; p.hd = hd; p.bs = bs;
   p.scale = scale; p.softcap = softcap; p.window = window;
   p.from_window = 0;
+  p.mask_chunk = mask_chunk; p.sink = sink ? 1 : 0; p.wide_weights = wide_weights ? 1 : 0;
   p.bs_shift = 0;
   while ((1 << p.bs_shift) < bs) p.bs_shift++;
   const float log2e = 1.4426950408889634f;
@@ -1199,8 +1255,10 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
       const int per_block = 4 * p.tpw;
       // no block of rows has more tiles than this, whatever its request's length
       int bound = (max_ctx + 31) / 32;
-      if (window > 0) bound = std::min(bound, (window + per_block + 31) / 32 + 1);
-      range_tiles = portion_ranges(max_q_len, max_ctx, window, per_block, nkv, r_prefill, bound);
+      // (a chunk's rows see no more keys than a window of its size would show them)
+      const int reach = mask_chunk > 0 ? mask_chunk : window;
+      if (reach > 0) bound = std::min(bound, (reach + per_block + 31) / 32 + 1);
+      range_tiles = portion_ranges(max_q_len, max_ctx, window, mask_chunk, per_block, nkv, r_prefill, bound);
       if (range_tiles) {
         most_ranges = (bound + range_tiles - 1) / range_tiles;
         if (R - r_prefill > 0) split_at = (zk_attention_bf16_workspace(R - r_prefill, nh, hd, max_ctx) + 255) / 256 * 256;
@@ -1252,8 +1310,9 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
       span = 4 * p.chunk;
       p.nchunks = grid.x;
       // a window covers at most ceil(window / span) + 1 blocks of span keys
-      const int window_blocks = window > 0 ? (window + span - 1) / span + 1 : 0;
-      if (window > 0 && window_blocks < (int)grid.x) {
+      const int reach = mask_chunk > 0 ? mask_chunk : window;
+      const int window_blocks = reach > 0 ? (reach + span - 1) / span + 1 : 0;
+      if (reach > 0 && window_blocks < (int)grid.x) {
         p.from_window = 1;
         grid.x = window_blocks;
       }
@@ -1272,12 +1331,27 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
     if (rc) return rc;
     dim3 cgrid(n_dec, nh);
     attn_combine_kernel<<<cgrid, 256, 0, s>>>(p.part_o, p.part_ml, q_start, ctx_len, (__bf16*)out, nh, hd,
-                                              window, r_prefill, p.nchunks, span);
+                                              window, r_prefill, p.nchunks, span, mask_chunk, sink);
     return zk_launch_status("zk_attention_bf16 (combine)");
   }
   return 0;
 }
 
+int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const void* vcache_t,
+                      const int* block_table, int max_blocks, const int* q_start, const int* ctx_len,
+                      void* out, int R, int r_prefill, int max_q_len, int max_ctx, int nh, int nkv,
+                      int hd, int bs, float scale, float softcap, int window, int decode_chunk,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+  return zk_attention_bf16_masked(q, q_stride, kcache, vcache_t, block_table, max_blocks, q_start, ctx_len, out, R,
+                                  r_prefill, max_q_len, max_ctx, nh, nkv, hd, bs, scale, softcap, window, decode_chunk,
+                                  workspace, workspace_bytes, 0, 0, 0, stream);
+}
+
 }  // extern "C"
+
+extern "C" int zk_steplist_register(const char* name, int nargs, void* fn);
+static const int zk_attention_bf16_masked_entered = zk_steplist_register(
+    "zk_attention_bf16_masked", zk_packed::Call<zk_attention_bf16_masked>::nargs,
+    (void*)zk_packed::Call<zk_attention_bf16_masked>::call);
 
 #endif  // ZSE_ACT_BF16

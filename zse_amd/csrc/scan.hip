@@ -43,6 +43,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(
   __shared__ __attribute__((aligned(16))) float Cs[GRP][NPAD];
   __shared__ float steps[GRP][SCAN_CHANNELS];
   __shared__ float us[GRP][SCAN_CHANNELS];
+  __shared__ float zs[GRP][SCAN_CHANNELS];         // the gate going in, the gated read-out coming back
   const int r = blockIdx.x, ch0 = blockIdx.y * SCAN_CHANNELS, tid = threadIdx.x;
   const int col = tid >> 2, j = tid & 3, c = ch0 + col;
   const int t0 = q_start[r], t1 = q_start[r + 1];
@@ -74,6 +75,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(
       const bool in = ch0 + cc < inner;
       steps[tt][cc] = in ? scan_softplus(dt[(size_t)(c0 + tt) * lddt + ch0 + cc] + dt_bias[ch0 + cc]) : 0.f;
       us[tt][cc] = in ? to_f32(u[(size_t)(c0 + tt) * ldu + ch0 + cc]) : 0.f;
+      zs[tt][cc] = in ? to_f32(z[(size_t)(c0 + tt) * ldz + ch0 + cc]) : 0.f;
     }
     __syncthreads();
     for (int tt = 0; tt < n_tok; tt++) {
@@ -95,10 +97,17 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(
         acc1 = fmaf(s[4 * i + 3], cv.w, acc1);
       }
       const float y = scan_sum4(acc0 + acc1) + dskip * x;
-      if (j == 0 && live) {
-        const float zz = to_f32(z[(size_t)(c0 + tt) * ldz + c]);
-        out[(size_t)(c0 + tt) * inner + c] = from_f32<act_t>(y * (zz / (1.0f + expf(-zz))));
+      // the walk touches no global memory: a channel's gate waits in local memory, and its
+      // result takes the gate's place (the channel's four lanes are in one wave)
+      if (j == 0) {
+        const float zz = zs[tt][col];
+        zs[tt][col] = y * (zz / (1.0f + expf(-zz)));
       }
+    }
+    __syncthreads();
+    for (int i = tid; i < n_tok * SCAN_CHANNELS; i += 256) {
+      const int tt = i / SCAN_CHANNELS, cc = i % SCAN_CHANNELS;
+      if (ch0 + cc < inner) out[(size_t)(c0 + tt) * inner + ch0 + cc] = from_f32<act_t>(zs[tt][cc]);
     }
   }
   if (live) {

@@ -192,7 +192,7 @@ def bumolix_plan(c: BumolixConfig) -> ModelPlan:
                 hidden_size=c.width, num_heads=a.heads, num_kv_heads=a.kv_heads, head_dim=a.dim, scale=a.scale,
                 softcap=None, window=None, position=rotary, names={r: lm + r for r in ("q", "k", "v", "o")},
                 value_dim=a.vdim, norm_eps=c.eps, biases={r: f"{lm}{r}.b" for r in ("q", "k", "v")}, chunk=a.chunk,
-                unit_sink=True, qk_unit_norm=True, gate=lm + "g")
+                unit_sink=True, qk_unit_norm=True, gate=lm + "g", wide_weights=True)
             right = LinearAttentionSpec(
                 hidden_size=c.width, num_heads=g.heads, key_dim=g.dim, value_dim=g.vdim, decay_rank=g.rank, tau=g.tau,
                 eps=c.eps, names={"q": rm + "q", "k": rm + "k", "v": rm + "v", "gate": rm + "g", "o": rm + "o",

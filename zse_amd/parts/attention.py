@@ -47,13 +47,14 @@ class PagedAttention(Part):
         self.unit_sink = bool(getattr(s, "unit_sink", False))
         self.unit_norm = bool(getattr(s, "qk_unit_norm", False))
         self.gate_name = getattr(s, "gate", None)
+        self.wide_weights = bool(getattr(s, "wide_weights", False))
         if self.chunk and s.window:
             raise ValueError("an attention has a window or a chunk, not both")
         if self.chunk < 0:
             raise ValueError(f"chunk must be positive, got {self.chunk}")
         self.general = bool(self.value_dim != s.head_dim or self.q_norm_name or self.k_norm_name or
                             self.head_scale_name or self.value_base or self.bias_names or
-                            self.rot_scale != 1.0 or self.rot_interleaved or self.chunk or self.unit_sink or
+                            self.rot_scale != 1.0 or self.rot_interleaved or self.chunk or self.unit_sink or self.wide_weights or
                             self.unit_norm or self.gate_name)
         self.in_bias = self.o_bias = None
         if self.value_dim > 256:
@@ -130,7 +131,7 @@ class PagedAttention(Part):
     def wants_v_transposed(self, kernels, dtype: str, page_size: int) -> bool:
         """The matrix-core kernel reads V as [page][kv head][hd][bs]."""
         s = self.spec
-        if (self.chunk or self.unit_sink) and not kernels.has("zk_attention_bf16_masked"):
+        if (self.chunk or self.unit_sink or self.wide_weights) and not kernels.has("zk_attention_bf16_masked"):
             return False
         return bool(dtype == BF16 and self.value_dim == s.head_dim and kernels.has("zk_attention_bf16") and
                     kernels.zk_attention_bf16_supports(s.num_heads, s.num_kv_heads, s.head_dim, page_size))
@@ -200,13 +201,13 @@ class PagedAttention(Part):
         o = ctx.alloc((T, nh * vd))
         cap = float(s.softcap) if s.softcap else 0.0
         win = int(s.window) if s.window else 0
-        masked = bool(self.chunk or self.unit_sink)
+        masked = bool(self.chunk or self.unit_sink or self.wide_weights)
         if masked and cache.v_transposed and ctx.tuned and vd == hd:
             k.zk_attention_bf16_masked(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
                                        ctx.q_start, ctx.ctx_len, o.ptr, ctx.R, ctx.n_multi, ctx.max_q_len,
                                        ctx.max_ctx, nh, nkv, hd, g.page_size, s.scale, cap, win,
                                        self.decode_chunk, ctx.workspace.ptr, ctx.workspace.nbytes, self.chunk,
-                                       1 if self.unit_sink else 0, ctx.stream)
+                                       1 if self.unit_sink else 0, 1 if self.wide_weights else 0, ctx.stream)
         elif masked:
             k.zk_attention_plain_masked(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
                                         ctx.req_of_token, ctx.positions, o.ptr, T, nh, nkv, hd, vd, g.page_size, s.scale,

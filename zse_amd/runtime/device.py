@@ -218,6 +218,8 @@ BF16_KERNEL_SIGNATURES = {
     "zk_qkv_rope_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "zk_attention_bf16": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
                           _F, _F, _I, _I, _VP, _SZ, _VP],
+    "zk_attention_bf16_masked": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
+                                 _F, _F, _I, _I, _VP, _SZ, _I, _I, _I, _VP],
     "zk_latent_attention_bf16": [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _SZ, _I, _I, _I, _I, _I, _I, _I, _I, _F, _VP],
     "zk_moe_experts_grouped": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP],
 }
