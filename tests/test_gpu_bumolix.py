@@ -259,6 +259,38 @@ def test_the_recurrence_remembers_the_first_tokens(tmp_path, kind, dtype):
         assert_close(rows["other"], ref_other, dtype, f"{how} other")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("segment", [16, 64])
+def test_long_portions_walked_in_segments(tmp_path, monkeypatch, segment, dtype):
+    """Few long portions: the recurrences walk segments of a portion side by side and join them.
+    Portions that end inside a segment, on its edge and one past it, beside a short one; later
+    portions start from the state the earlier ones left; decays near one and far from it."""
+    from zse_amd.parts.gla import GatedLinearAttention
+    from zse_amd.parts.scan import SelectiveScan
+    monkeypatch.setattr(GatedLinearAttention, "SEGMENT", segment)
+    monkeypatch.setattr(SelectiveScan, "SEGMENT", segment)
+    cfg = config([parallel_layer(left(2, 1, 8, 8, chunk=24, rot_dims=4), right(3, 12, 40, 2.0, 4), 0.6, 1.4, dense(24)),
+                  scan_layer(72, 5, 3, 3, None),
+                  parallel_layer(left(1, 1, 16, 16, chunk=9, rot_dims=8), right(1, 40, 24, 9.0, 2), 1.0, 1.0, None)],
+                 vocab=70, width=40, mult=0.6)
+    w = random_weights(cfg, 31)
+    w["l0.mix.right.a2.b"][:] = np.linspace(-4.0, 8.0, 36)
+    w["l1.mix.A_log"][:] = np.linspace(-5.0, 1.5, 72 * 5).reshape(72, 5)
+    lengths = {"a": 4 * segment + 7, "b": 2 * segment, "c": 2 * segment + 1, "d": 5, "e": 3 * segment - 1}
+    streams = {r: tokens_of(cfg["vocab"], n, 60 + i) for i, (r, n) in enumerate(lengths.items())}
+    refs = {r: P.forward(cfg, w, t, np.float64) for r, t in streams.items()}
+    folder = write_model(str(tmp_path / f"segments_{segment}_{dtype}"), cfg, w, dtype)
+    runner = make_runner(folder, dtype, page_size=8, cache_tokens=1024, max_seqs=3, max_batch_tokens=1024, max_model_len=512)
+    check(run_steps(runner, streams, whole_steps(streams)), refs, dtype, "whole")
+    # a, b and d in one step, then c and e with what is left of nothing: three requests of unequal length a step
+    together = [([("a", lengths["a"]), ("b", lengths["b"]), ("d", lengths["d"])], ["a", "b", "d"]),
+                ([("c", lengths["c"]), ("e", lengths["e"])], ["c", "e"])]
+    check(run_steps(runner, streams, together), refs, dtype, "unequal requests together")
+    sizes = (2 * segment + 3, 2, 2 * segment, 1, 3 * segment)
+    check(run_steps(runner, streams, chunked_steps(streams, sizes=sizes)), refs, dtype, "long portions one after the other")
+    assert runner.manager.slots.free_slots == 3
+
+
 def test_decays_far_from_one_and_steps_of_every_size(tmp_path):
     """tau = 1 with strongly negative arguments forgets within a token or two, large steps of the
     scan saturate exp(step A): the 32-bit arithmetic of decays, logarithms and softplus holds at

@@ -17,6 +17,14 @@
 // blocks leaves that to a second kernel).  Every sum runs in an order fixed by the channel
 // numbers alone, so a request's values are the same bits however its tokens are cut into steps.
 // All arithmetic is float; q, k, v, g come in the activation type, z as floats.
+//
+// Few requests with long portions leave most of the chip idle on such a walk, and the recurrence is
+// linear in S: a portion is then cut into segments of seg_len tokens that are walked side by side,
+// twice.  The first walk starts every segment from zero and keeps what it adds, L_s, and the
+// product of its decays, P_s; a small kernel goes through the segments in order (start_0 = S,
+// start_(s+1) = diag(P_s) start_s + L_s) and leaves every segment its starting state; the second
+// walk starts from those, reads out, and its last segment stores the request's state.  The sums
+// are the same, grouped by segments, so the values differ from the plain walk's by rounding alone.
 #include "common.h"
 #include "packed_call.h"
 
@@ -52,29 +60,47 @@ __global__ __launch_bounds__(1024) void gla_kernel(
     const float* __restrict__ z, int ldz, const float* __restrict__ z_bias, float inv_tau,
     const float* __restrict__ gain, float* __restrict__ state, int slot_words, int offset_words,
     const int* __restrict__ q_start, const int* __restrict__ slot_of_req, act_t* __restrict__ out,
-    float* __restrict__ raw, int H, int D, int E, float eps, float q_scale, int COLS) {
+    float* __restrict__ raw, int H, int D, int E, float eps, float q_scale, int COLS, int mode, int seg_len, int nseg,
+    float* __restrict__ seg_state, float* __restrict__ seg_decay) {
   constexpr int DMAX = 4 * CH * DS, RD = 4 * CH, GRP = GLA_GROUP;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* qs = lds;                                 // [GRP][DMAX]
   float* ks = qs + GRP * DMAX;                     // [GRP][DMAX]
   float* as = ks + GRP * DMAX;                     // [GRP][DMAX]: the decays
   float* ov = as + GRP * DMAX;                     // [GRP][COLS]: v going in, the read-out coming back
-  const int r = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * COLS, tid = threadIdx.x, nt = blockDim.x;
+  float* prod = ov + GRP * COLS;                   // [DMAX]: the product of a segment's decays (mode 1)
+  // mode 0: the plain walk, nseg == 1.  mode 1: a segment from zero, its sum and decays kept.
+  // mode 2: a segment from its starting state, read out.
+  const int r = blockIdx.x / nseg, seg = blockIdx.x - r * nseg;
+  const int h = blockIdx.y, e0 = blockIdx.z * COLS, tid = threadIdx.x, nt = blockDim.x;
   const int lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
   const int col = tid / DS, j = tid % DS, e = e0 + col;
-  const int t0 = q_start[r], t1 = q_start[r + 1];
+  int t0 = q_start[r], t1 = q_start[r + 1];
   if (t1 <= t0) return;
+  bool last_seg = true;
+  if (mode != 0) {
+    const int segs = (t1 - t0 + seg_len - 1) / seg_len;
+    last_seg = seg == segs - 1;
+    if (seg >= segs || (mode == 1 && last_seg)) return;        // nothing follows the last segment
+    t0 += seg * seg_len;
+    t1 = min(t1, t0 + seg_len);
+  }
   const bool live = e < E;
+  const bool readout = mode != 1;
   const int cols = min(COLS, E - e0);
   float* S = state + (size_t)slot_of_req[r] * slot_words + offset_words + (size_t)h * D * E;
+  float* Sseg = mode != 0 ? seg_state + ((size_t)blockIdx.x * H + h) * D * E : nullptr;
+  const float* Sfrom = mode == 2 ? Sseg : S;
   float s[RD];
 #pragma unroll
   for (int i = 0; i < CH; i++)
 #pragma unroll
     for (int c = 0; c < 4; c++) {
       const int d = 4 * (j + DS * i) + c;
-      s[4 * i + c] = (live && d < D) ? S[(size_t)d * E + e] : 0.f;
+      s[4 * i + c] = (mode != 1 && live && d < D) ? Sfrom[(size_t)d * E + e] : 0.f;
     }
+  if (mode == 1)
+    for (int d = tid; d < DMAX; d += nt) prod[d] = 1.f;
   for (int c0 = t0; c0 < t1; c0 += GRP) {
     const int n = min(GRP, t1 - c0);
     __syncthreads();
@@ -92,6 +118,12 @@ __global__ __launch_bounds__(1024) void gla_kernel(
       ov[i] = c < cols ? to_f32(qkv[(size_t)(c0 + tt) * ld + v_off + (size_t)h * E + e0 + c]) : 0.f;
     }
     __syncthreads();
+    if (mode == 1 && blockIdx.z == 0)
+      for (int d = tid; d < DMAX; d += nt) {
+        float pr = prod[d];
+        for (int tt = 0; tt < n; tt++) pr *= as[tt * DMAX + d];
+        prod[d] = pr;
+      }
     // the walk: no barrier.  What the next token needs (its k, decays and v) is asked for before this
     // token's arithmetic.
     float4 kn[CH], an[CH];
@@ -133,6 +165,10 @@ __global__ __launch_bounds__(1024) void gla_kernel(
         s[4 * i + 1] = fmaf(s[4 * i + 1], aa[i].y, kk[i].y * vt);
         s[4 * i + 2] = fmaf(s[4 * i + 2], aa[i].z, kk[i].z * vt);
         s[4 * i + 3] = fmaf(s[4 * i + 3], aa[i].w, kk[i].w * vt);
+      }
+      if (!readout) continue;
+#pragma unroll
+      for (int i = 0; i < CH; i++) {
         a0 = fmaf(s[4 * i], qq[i].x, a0);
         a1 = fmaf(s[4 * i + 1], qq[i].y, a1);
         a2 = fmaf(s[4 * i + 2], qq[i].z, a2);
@@ -144,6 +180,7 @@ __global__ __launch_bounds__(1024) void gla_kernel(
       if (j == 0) ov[tt * COLS + col] = o;
     }
     __syncthreads();
+    if (!readout) continue;
     if (raw != nullptr) {                          // the head spans several blocks: its norm comes later
       for (int i = tid; i < n * COLS; i += nt) {
         const int tt = i / COLS, c = i % COLS;
@@ -164,14 +201,44 @@ __global__ __launch_bounds__(1024) void gla_kernel(
       }
     }
   }
-  if (live) {
+  if (mode == 1 && blockIdx.z == 0)                // written by the threads that made them
+    for (int d = tid; d < D; d += nt) seg_decay[((size_t)blockIdx.x * H + h) * D + d] = prod[d];
+  float* Sto = mode == 1 ? Sseg : S;
+  if (live && (mode != 2 || last_seg)) {
 #pragma unroll
     for (int i = 0; i < CH; i++)
 #pragma unroll
       for (int c = 0; c < 4; c++) {
         const int d = 4 * (j + DS * i) + c;
-        if (d < D) S[(size_t)d * E + e] = s[4 * i + c];
+        if (d < D) Sto[(size_t)d * E + e] = s[4 * i + c];
       }
+  }
+}
+
+// Through a request's segments in order: what a segment added from zero gives way to the state
+// it starts from.  One thread an element of S; the last segment adds nothing here (it stores the
+// request's state itself, after its second walk).
+__global__ __launch_bounds__(256) void gla_segments_kernel(
+    float* __restrict__ seg_state, const float* __restrict__ seg_decay, const float* __restrict__ state, int slot_words,
+    int offset_words, const int* __restrict__ q_start, const int* __restrict__ slot_of_req, int seg_len, int nseg,
+    int H, int D, int E) {
+  const int r = blockIdx.y;
+  const int n_tok = q_start[r + 1] - q_start[r];
+  if (n_tok <= 0) return;
+  const int segs = (n_tok + seg_len - 1) / seg_len;
+  const size_t per = (size_t)H * D * E;
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= per) return;
+  const size_t hd = i / E;                         // h * D + d
+  float cur = state[(size_t)slot_of_req[r] * slot_words + offset_words + i];
+  float* ss = seg_state + (size_t)r * nseg * per + i;
+  const float* pd = seg_decay + (size_t)r * nseg * H * D + hd;
+  for (int sg = 0; sg < segs; sg++) {
+    const bool more = sg + 1 < segs;
+    const float added = more ? ss[(size_t)sg * per] : 0.f;
+    const float decay = more ? pd[(size_t)sg * H * D] : 0.f;
+    ss[(size_t)sg * per] = cur;
+    cur = fmaf(decay, cur, added);
   }
 }
 
@@ -211,7 +278,7 @@ extern "C" {
 int zk_gla(const void* qkv, int ld, int k_off, int v_off, const void* g, int ldg, const float* z, int ldz,
            const float* z_bias, float tau, const float* gain, float* state, int slot_words, int offset_words,
            const int* q_start, const int* slot_of_req, const int* positions, void* out, float* raw, int T, int R,
-           int max_q_len, int H, int D, int E, float eps, void* stream) {
+           int max_q_len, int H, int D, int E, float eps, int seg_len, float* seg_state, float* seg_decay, void* stream) {
   ZK_REQUIRE(T >= 0 && R >= 0 && H > 0 && D > 0 && E > 0 && tau > 0.f, "zk_gla: bad sizes");
   ZK_REQUIRE(D <= 256, "zk_gla: up to 256 query/key channels a head");
   ZK_REQUIRE(H <= 65535 && (E + GLA_COLS_LONG - 1) / GLA_COLS_LONG <= 65535, "zk_gla: too many heads or value channels");
@@ -228,18 +295,37 @@ int zk_gla(const void* qkv, int ld, int k_off, int v_off, const void* g, int ldg
   const int unit = 64 / DS;                                             // columns of a wave
   const int cols = E < per_block ? (E + unit - 1) / unit * unit : per_block;
   const int threads = cols * DS;
-  const size_t lds = (size_t)GLA_GROUP * (3 * DMAX + cols) * sizeof(float);
-  dim3 grid(R, H, blocks_e);
+  const size_t lds = (size_t)GLA_GROUP * (3 * DMAX + cols) * sizeof(float) + DMAX * sizeof(float);
+  // segments: seg_state float [R * nseg, H * D * E], seg_decay float [R * nseg, H * D], nseg as below
+  const bool segmented = seg_len > 0 && seg_state != nullptr && seg_decay != nullptr && max_q_len > seg_len;
+  ZK_REQUIRE(seg_len <= 0 || seg_len % GLA_GROUP == 0, "zk_gla: segments of whole groups of tokens");
+  const int nseg = segmented ? (max_q_len + seg_len - 1) / seg_len : 1;
+  ZK_REQUIRE((long long)R * nseg <= 0x7fffffffLL / 2, "zk_gla: too many segments");
+  dim3 grid(R * nseg, H, blocks_e);
   float* raw_arg = blocks_e > 1 ? raw : nullptr;
   const float q_scale = 1.0f / sqrtf((float)D);
-#define LAUNCH(C, L)                                                                                              \
+#define LAUNCH(C, L, MODE)                                                                                        \
   gla_kernel<C, L><<<grid, threads, lds, (hipStream_t)stream>>>(                                                  \
       (const act_t*)qkv, ld, k_off, v_off, (const act_t*)g, ldg, z, ldz, z_bias, 1.0f / tau, gain, state,        \
-      slot_words, offset_words, q_start, slot_of_req, (act_t*)out, raw_arg, H, D, E, eps, q_scale, cols)
-  if (DMAX == 32) LAUNCH(1, 8);
-  else if (DMAX == 64) LAUNCH(2, 8);
-  else if (DMAX == 128) LAUNCH(4, 8);
-  else LAUNCH(4, 16);
+      slot_words, offset_words, q_start, slot_of_req, (act_t*)out, raw_arg, H, D, E, eps, q_scale, cols, MODE,   \
+      seg_len, nseg, seg_state, seg_decay)
+#define WALK(MODE)                                                                                                \
+  do {                                                                                                            \
+    if (DMAX == 32) LAUNCH(1, 8, MODE);                                                                           \
+    else if (DMAX == 64) LAUNCH(2, 8, MODE);                                                                      \
+    else if (DMAX == 128) LAUNCH(4, 8, MODE);                                                                     \
+    else LAUNCH(4, 16, MODE);                                                                                     \
+  } while (0)
+  if (segmented) {
+    WALK(1);
+    dim3 sg((unsigned)(((size_t)H * D * E + 255) / 256), R);
+    gla_segments_kernel<<<sg, 256, 0, (hipStream_t)stream>>>(seg_state, seg_decay, state, slot_words, offset_words,
+                                                             q_start, slot_of_req, seg_len, nseg, H, D, E);
+    WALK(2);
+  } else {
+    WALK(0);
+  }
+#undef WALK
 #undef LAUNCH
   if (blocks_e > 1) {
     dim3 fg(T, H);

@@ -11,7 +11,10 @@ carried as floats in the request's state slot:
 
 q, k, v, the gate and the narrow W_a1 are one product; W_a2 reads the last of its columns and
 leaves floats.  One kernel walks the tokens of every (request, head), so steps of single tokens
-and portions of prompts run the same arithmetic in the same order.
+and portions of prompts run the same arithmetic in the same order.  Where few long portions
+would leave most of the chip idle, the kernel walks segments of a portion side by side (twice:
+what each adds from zero, then, from the starting states that follow, the read-outs): the same
+sums grouped by segments.
 """
 from __future__ import annotations
 
@@ -24,6 +27,8 @@ from .ops import linear
 
 class GatedLinearAttention(Part):
     graph_safe = True      # rows, requests and slots are read by the kernels from device memory
+    SEGMENT = 64           # tokens of a segment of a long portion
+    ENOUGH_BLOCKS = 1024   # a plain walk with this many blocks fills the chip without segments
 
     def __init__(self, spec):
         s = self.spec = spec
@@ -78,10 +83,16 @@ class GatedLinearAttention(Part):
         out = ctx.alloc((T, self.vv))
         # read-outs before their norm, for steps in which a head's value channels spread over several blocks
         raw = ctx.alloc((T, self.vv), F32) if (E > 64 or ctx.max_q_len > 16) else None
+        seg_len, seg_state, seg_decay = 0, None, None
+        if raw is not None and ctx.max_q_len >= 2 * self.SEGMENT and ctx.R * H * -(-E // 16) < self.ENOUGH_BLOCKS:
+            seg_len = self.SEGMENT
+            segs = ctx.R * -(-int(ctx.max_q_len) // seg_len)
+            seg_state = ctx.alloc((segs, self.state_words()), F32).ptr
+            seg_decay = ctx.alloc((segs, self.qk), F32).ptr
         k.zk_gla(rows.ptr, ld, self.qk, 2 * self.qk, rows.ptr + (2 * self.qk + self.vv) * item, ld, z.ptr, self.qk,
                  self.a_bias.ptr, float(s.tau), self.gain.ptr, ctx.state.ptr, ctx.state.shape[1], cache.state_offset // 4,
                  ctx.q_start, ctx.slot_of_req, ctx.positions, out.ptr, raw.ptr if raw is not None else None, T, ctx.R,
-                 int(ctx.max_q_len), H, D, E, float(s.eps), ctx.stream)
+                 int(ctx.max_q_len), H, D, E, float(s.eps), seg_len, seg_state, seg_decay, ctx.stream)
         return linear(ctx, out, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)
 
 

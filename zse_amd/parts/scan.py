@@ -23,6 +23,8 @@ from .ops import linear
 
 class SelectiveScan(Part):
     graph_safe = True      # rows, requests and slots are read by the kernels from device memory
+    SEGMENT = 64           # tokens of a segment of a long portion
+    ENOUGH_BLOCKS = 1024   # a plain walk with this many blocks fills the chip without segments
 
     def __init__(self, spec):
         s = self.spec = spec
@@ -76,9 +78,17 @@ class SelectiveScan(Part):
         p = linear(ctx, u, self.w_x, ctx.alloc((T, ldp)))
         dt = linear(ctx, Tensor(p.ptr, (T, R), ctx.dtype, p.owner), self.w_dt, ctx.alloc((T, I), F32), lda=ldp)
         out = ctx.alloc((T, I))
+        # few long portions: segments of a portion walked side by side (see the kernel's file)
+        seg_len, seg_state, seg_steps = 0, None, None
+        if ctx.max_q_len >= 2 * self.SEGMENT and ctx.R * -(-I // 64) < self.ENOUGH_BLOCKS:
+            seg_len = self.SEGMENT
+            segs = ctx.R * -(-int(ctx.max_q_len) // seg_len)
+            seg_state = ctx.alloc((segs, self.state_words()), F32).ptr
+            seg_steps = ctx.alloc((segs, I), F32).ptr
         k.zk_selective_scan(u.ptr, I, dt.ptr, I, self.dt_bias.ptr, p.ptr, ldp, R, R + N, self.A_log.ptr, self.D.ptr,
                             uz.ptr + I * item, 2 * I, ctx.state.ptr, ctx.state.shape[1], cache.state_offset // 4,
-                            ctx.q_start, ctx.slot_of_req, out.ptr, T, ctx.R, I, N, ctx.stream)
+                            ctx.q_start, ctx.slot_of_req, out.ptr, T, ctx.R, I, N, int(ctx.max_q_len), seg_len,
+                            seg_state, seg_steps, ctx.stream)
         return linear(ctx, out, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)
 
 

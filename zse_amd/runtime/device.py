@@ -204,9 +204,9 @@ KERNEL_SIGNATURES = {
     "zk_unary_act": [_VP, _VP, _SZ, _I, _VP],
     "zk_gate_heads": [_VP, _VP, _I, _I, _I, _VP],
     "zk_gla": [_VP, _I, _I, _I, _VP, _I, _VP, _I, _VP, _F, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I,
-               _F, _VP],
+               _F, _I, _VP, _VP, _VP],
     "zk_selective_scan": [_VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I,
-                          _I, _VP],
+                          _I, _I, _I, _VP, _VP, _VP],
 }
 # present only in the bf16 library
 BF16_KERNEL_SIGNATURES = {
