@@ -144,9 +144,12 @@ def attention_alone(chunk, dtype, tmp_path, right_scale=0.0, **kw):
     return cfg, w, write_model(str(tmp_path / f"alone_{chunk}_{dtype}"), cfg, w, dtype)
 
 
+# head shapes: values of another size than keys run on the plain attention kernel in either type,
+# equal sizes of 16, 32, ... on the matrix-core kernel in bfloat16 (the far key of this draw shows with heads of 16)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_key_hundreds_of_tokens_back_in_its_chunk(tmp_path, dtype):
-    cfg, w, folder = attention_alone(400, dtype, tmp_path)
+@pytest.mark.parametrize("dim,vdim", [(16, 24), (16, 16)])
+def test_a_key_hundreds_of_tokens_back_in_its_chunk(tmp_path, dim, vdim, dtype):
+    cfg, w, folder = attention_alone(400, dtype, tmp_path, dim=dim, vdim=vdim)
     n = 390
     base = tokens_of(cfg["vocab"], n, 21)
     ref = P.forward(cfg, w, base, np.float64)
@@ -172,13 +175,14 @@ def test_a_key_hundreds_of_tokens_back_in_its_chunk(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("vdim", [24, 16])
 @pytest.mark.parametrize("chunk,page", [(12, 8), (7, 4), (40, 16), (16, 16), (33, 4)])
-def test_keys_just_inside_and_just_outside_a_chunks_edge(tmp_path, chunk, page, dtype):
+def test_keys_just_inside_and_just_outside_a_chunks_edge(tmp_path, chunk, page, vdim, dtype):
     """With the attention alone, a change of the last token before a chunk must leave every logit
     of the chunk as it was, to the bit, and a change of the chunk's first token must move them
     as the plain implementation says; in prompts, in portions that end and begin at and around
     the edge, and token by token."""
-    cfg, w, folder = attention_alone(chunk, dtype, tmp_path)
+    cfg, w, folder = attention_alone(chunk, dtype, tmp_path, vdim=vdim)
     n = 3 * chunk + chunk // 2
     base = tokens_of(cfg["vocab"], n, 3)
     edge = 2 * chunk
@@ -204,11 +208,12 @@ def test_keys_just_inside_and_just_outside_a_chunks_edge(tmp_path, chunk, page, 
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_the_sink_takes_its_share_of_the_weights(tmp_path, dtype):
+@pytest.mark.parametrize("vdim", [8, 16])
+def test_the_sink_takes_its_share_of_the_weights(tmp_path, vdim, dtype):
     """Scores of either sign and several units: a query whose keys all score low gives most of its
     weight to the sink, one with a high score nearly nothing.  Left out of the denominator, or
     given a value, the sink would move every such row."""
-    cfg, w, folder = attention_alone(9, dtype, tmp_path, scale=0.5, heads=3, kv_heads=3, vdim=8)
+    cfg, w, folder = attention_alone(9, dtype, tmp_path, scale=0.5, heads=3, kv_heads=3, vdim=vdim)
     toks = tokens_of(cfg["vocab"], 50, 5)
     x = P.rms_norm(w["embed"][toks].astype(np.float64), w["l0.norm1"], cfg["norm"]["eps"], np.float64)
     m = cfg["layers"][0]["mixer"]["left"]

@@ -53,7 +53,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // <= 0: none) and that value's column in ``partials`` [M][strips] as (float, int), larger value
 // first, equal values to the lower column, NaN never, which a joining kernel reduces to one
 // column a row: the greedy choice without the logits ever reaching memory.
-enum { EPI_NONE = 0, EPI_SOFTCAP = 1, EPI_GELU_TANH = 2, EPI_SILU = 3, EPI_PICK = 4, EPI_RELU = 5, EPI_CLAMPED = 6 };
+enum { EPI_NONE = 0, EPI_SOFTCAP = 1, EPI_GELU_TANH = 2, EPI_SILU = 3, EPI_PICK = 4, EPI_RELU = 5, EPI_CLAMPED = 6, EPI_RELU2 = 7 };
 
 struct Pick {
   float value;
@@ -85,6 +85,17 @@ __device__ __forceinline__ Pick pick_of_strip(const float (&x)[4], int n, int N,
     }
   }
   return p;
+}
+
+// What a plain (not gated) product does to a sum before it is stored: the soft cap, the square of
+// relu, or nothing.
+__device__ __forceinline__ float epi_unary(float x, int epi, float cap) {
+  if (epi == EPI_SOFTCAP) return cap * tanhf(x / cap);
+  if (epi == EPI_RELU2) {
+    const float r = fmaxf(x, 0.f);
+    return r * r;
+  }
+  return x;
 }
 
 // 0.5 g (1 + tanh(u)) = g / (1 + exp(-2 u)): one exponential and one reciprocal instead of the
@@ -382,7 +393,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
       if (n >= N) continue;
       float x = v[0][i];
       if (GATED) x = epi_gate(x, v[NS - 1][i], epi, cap);
-      else if (epi == EPI_SOFTCAP) x = cap * tanhf(x / cap);
+      else x = epi_unary(x, epi, cap);
       if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
       else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
     }
@@ -431,7 +442,7 @@ __device__ __forceinline__ void tile_store_quad(const f32x4& x0, const f32x4& x1
         const int n = n0 + wn * 64 + j * 32 + c;
         if (n >= N) continue;
         float x = j ? x1[e] : x0[e];
-        if (epi == EPI_SOFTCAP) x = cap * tanhf(x / cap);
+        x = epi_unary(x, epi, cap);
         if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
         else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
       }
@@ -472,9 +483,9 @@ __device__ __forceinline__ void tile_store_staged(const f32x16 (&acc)[WMT][2], _
         x[e] = acc[i][0][4 * b + e];
         y[e] = acc[i][1][4 * b + e];
         if (GATED) x[e] = epi_gate(x[e], y[e], epi, cap);
-        else if (epi == EPI_SOFTCAP) {
-          x[e] = cap * tanhf(x[e] / cap);
-          y[e] = cap * tanhf(y[e] / cap);
+        else {
+          x[e] = epi_unary(x[e], epi, cap);
+          y[e] = epi_unary(y[e], epi, cap);
         }
       }
       __bf16* dst = stage + (i * 32 + lr) * SLD + 8 * b + 4 * lk;
@@ -862,7 +873,7 @@ __global__ __launch_bounds__(256) void gemm_tile_join_kernel(
     // time, half a line's bytes from one wave and the other half from another).  The block's
     // 256 threads are (b, lr, j) here; the sums are the same, in the same order.
     const int m0 = tm * BM + (wave / NWN) * (32 * WMT) + i * 32, n0 = tn * BN + (wave % NWN) * 64;
-    if (!c_is_f32 && epi == EPI_NONE && ldc % 8 == 0 && (uintptr_t)C % 16 == 0 && m0 + 32 <= M && n0 + 64 <= N) {
+    if (!c_is_f32 && (epi == EPI_NONE || epi == EPI_RELU2) && ldc % 8 == 0 && (uintptr_t)C % 16 == 0 && m0 + 32 <= M && n0 + 64 <= N) {
       const int lr = lane & 31, j = lane >> 5;
       const f32x4* at = partials + ((size_t)tile * ksplit * NW + wave) * per_wave + ((size_t)(i * 2 + j) * 64 + lr) * 4 + b;
       f32x4 lo = at[0], hi = at[32 * 4];
@@ -873,8 +884,8 @@ __global__ __launch_bounds__(256) void gemm_tile_join_kernel(
       bf16x8 out;
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        out[e] = (__bf16)lo[e];
-        out[4 + e] = (__bf16)hi[e];
+        out[e] = (__bf16)epi_unary(lo[e], epi, cap);
+        out[4 + e] = (__bf16)epi_unary(hi[e], epi, cap);
       }
       *(bf16x8*)((__bf16*)C + (size_t)(m0 + lr) * ldc + n0 + j * 32 + 8 * b) = out;
       return;
@@ -991,7 +1002,7 @@ __device__ __forceinline__ void mid_store(const f32x4 (&acc)[GATED ? 2 : 1][MT],
       if (n >= N) continue;
       float x = acc[0][mt][i];
       if (GATED) x = epi_gate(x, acc[GATED ? 1 : 0][mt][i], epi, cap);
-      else if (epi == EPI_SOFTCAP) x = cap * tanhf(x / cap);
+      else x = epi_unary(x, epi, cap);
       if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
       else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
     }
@@ -1162,7 +1173,7 @@ __global__ __launch_bounds__(256) void gemm_join_kernel(const float* __restrict_
     if (n + i >= N) continue;
     float v = x[i];
     if (GATED) v = epi_gate(v, y[i], epi, cap);
-    else if (epi == EPI_SOFTCAP) v = cap * tanhf(v / cap);
+    else v = epi_unary(v, epi, cap);
     if (c_is_f32) ((float*)C)[(size_t)m * ldc + n + i] = v;
     else ((__bf16*)C)[(size_t)m * ldc + n + i] = (__bf16)v;
   }
@@ -1429,7 +1440,7 @@ static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc
   ZK_REQUIRE(M >= 0 && N > 0 && K > 0, "zk_gemm_bf16: bad sizes");
   ZK_REQUIRE(K % 8 == 0 && lda % 8 == 0, "zk_gemm_bf16: K and lda must be multiples of 8");
   ZK_REQUIRE(lda >= K && ldc >= N, "zk_gemm_bf16: leading dimensions too small");
-  ZK_REQUIRE(epi >= 0 && epi <= EPI_CLAMPED, "zk_gemm_bf16: unknown epilogue");
+  ZK_REQUIRE(epi >= 0 && epi <= EPI_RELU2, "zk_gemm_bf16: unknown epilogue");
   ZK_REQUIRE((epi != EPI_SOFTCAP && epi != EPI_CLAMPED) || cap > 0.f, "zk_gemm_bf16: soft cap or clamp limit must be positive");
   ZK_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "zk_gemm_bf16: operands must be 16-byte aligned");
   const bool gated = epi == EPI_GELU_TANH || epi == EPI_SILU || epi == EPI_RELU || epi == EPI_CLAMPED;

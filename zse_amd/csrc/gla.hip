@@ -61,7 +61,7 @@ __global__ __launch_bounds__(1024) void gla_kernel(
     const float* __restrict__ gain, float* __restrict__ state, int slot_words, int offset_words,
     const int* __restrict__ q_start, const int* __restrict__ slot_of_req, act_t* __restrict__ out,
     float* __restrict__ raw, int H, int D, int E, float eps, float q_scale, int COLS, int mode, int seg_len, int nseg,
-    float* __restrict__ seg_state, float* __restrict__ seg_decay) {
+    float* __restrict__ seg_state, float* __restrict__ seg_decay, int decays_ready) {
   constexpr int DMAX = 4 * CH * DS, RD = 4 * CH, GRP = GLA_GROUP;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* qs = lds;                                 // [GRP][DMAX]
@@ -108,10 +108,11 @@ __global__ __launch_bounds__(1024) void gla_kernel(
       const int tt = i / DMAX, d = i % DMAX;
       const act_t* row = qkv + (size_t)(c0 + tt) * ld + (size_t)h * D;
       const bool in = d < D;
-      qs[i] = in ? to_f32(row[d]) * q_scale : 0.f;
+      if (readout) qs[i] = in ? to_f32(row[d]) * q_scale : 0.f;
       ks[i] = in ? to_f32(row[k_off + d]) : 0.f;
       // padding rows of S stay zero whatever their decay
-      as[i] = in ? expf(log_sigmoid_f(z[(size_t)(c0 + tt) * ldz + (size_t)h * D + d] + z_bias[(size_t)h * D + d]) * inv_tau) : 0.f;
+      const float zz = in ? z[(size_t)(c0 + tt) * ldz + (size_t)h * D + d] : 0.f;
+      as[i] = !in ? 0.f : decays_ready ? zz : expf(log_sigmoid_f(zz + z_bias[(size_t)h * D + d]) * inv_tau);
     }
     for (int i = tid; i < n * COLS; i += nt) {
       const int tt = i / COLS, c = i % COLS;
@@ -215,6 +216,17 @@ __global__ __launch_bounds__(1024) void gla_kernel(
   }
 }
 
+// The decays of a step with long portions, made once where every block of a head and both walks
+// of a segment would make them again: z <- sigmoid(z + bias)^(1 / tau), the very expression of the walk.
+__global__ __launch_bounds__(256) void gla_decays_kernel(float* __restrict__ z, int ldz, const float* __restrict__ z_bias,
+                                                         float inv_tau, int T, int HD) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)T * HD) return;
+  const size_t t = i / HD, c = i - t * HD;
+  float* at = z + t * ldz + c;
+  *at = expf(log_sigmoid_f(*at + z_bias[c]) * inv_tau);
+}
+
 // Through a request's segments in order: what a segment added from zero gives way to the state
 // it starts from.  One thread an element of S; the last segment adds nothing here (it stores the
 // request's state itself, after its second walk).
@@ -268,14 +280,15 @@ extern "C" {
 
 // qkv: [T, ld] activations: H query heads of D at column 0, H key heads at k_off, H value heads of E
 // at v_off.  g: [T, ldg], H heads of E (the output gate before its silu).  z: float [T, ldz], H heads
-// of D (the decays before bias, sigmoid and root); z_bias: float [H * D]; gain: float [E].
+// of D (the decays before bias, sigmoid and root; overwritten with the decays where the step is walked in
+// segments); z_bias: float [H * D]; gain: float [E].
 // state: request r's S [H, D, E] lies at state[slot_of_req[r] * slot_words + offset_words].
 // out: [T, H * E].  Requests are rows [q_start[r], q_start[r + 1]).  raw: float scratch [T, H * E],
 // used by heads that span several blocks (may be null: a head of up to 128 value channels then
 // stays in one block whatever the step); positions: [T].  max_q_len: the longest portion of the
 // step: with long portions a block takes 16 value channels, so that a head's walk spreads over
 // more compute units.
-int zk_gla(const void* qkv, int ld, int k_off, int v_off, const void* g, int ldg, const float* z, int ldz,
+int zk_gla(const void* qkv, int ld, int k_off, int v_off, const void* g, int ldg, float* z, int ldz,
            const float* z_bias, float tau, const float* gain, float* state, int slot_words, int offset_words,
            const int* q_start, const int* slot_of_req, const int* positions, void* out, float* raw, int T, int R,
            int max_q_len, int H, int D, int E, float eps, int seg_len, float* seg_state, float* seg_decay, void* stream) {
@@ -308,7 +321,7 @@ int zk_gla(const void* qkv, int ld, int k_off, int v_off, const void* g, int ldg
   gla_kernel<C, L><<<grid, threads, lds, (hipStream_t)stream>>>(                                                  \
       (const act_t*)qkv, ld, k_off, v_off, (const act_t*)g, ldg, z, ldz, z_bias, 1.0f / tau, gain, state,        \
       slot_words, offset_words, q_start, slot_of_req, (act_t*)out, raw_arg, H, D, E, eps, q_scale, cols, MODE,   \
-      seg_len, nseg, seg_state, seg_decay)
+      seg_len, nseg, seg_state, seg_decay, segmented ? 1 : 0)
 #define WALK(MODE)                                                                                                \
   do {                                                                                                            \
     if (DMAX == 32) LAUNCH(1, 8, MODE);                                                                           \
@@ -317,6 +330,9 @@ int zk_gla(const void* qkv, int ld, int k_off, int v_off, const void* g, int ldg
     else LAUNCH(4, 16, MODE);                                                                                     \
   } while (0)
   if (segmented) {
+    // z is the caller's scratch: its rows become the decays themselves
+    gla_decays_kernel<<<(unsigned)(((size_t)T * H * D + 255) / 256), 256, 0, (hipStream_t)stream>>>(z, ldz, z_bias, 1.0f / tau,
+                                                                                                   T, H * D);
     WALK(1);
     dim3 sg((unsigned)(((size_t)H * D * E + 255) / 256), R);
     gla_segments_kernel<<<sg, 256, 0, (hipStream_t)stream>>>(seg_state, seg_decay, state, slot_words, offset_words,

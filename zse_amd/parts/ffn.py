@@ -98,7 +98,7 @@ class MLP(Part):
     def forward(self, ctx, x: Tensor) -> Tensor:
         s = self.spec
         T, I = x.shape[0], s.intermediate_size
-        if tuned_gemm(ctx, s.hidden_size) and ctx.k.has("zk_gemm_bf16_unary"):
+        if tuned_gemm(ctx, s.hidden_size) and x.ptr % 16 == 0:
             a = linear(ctx, x, self.w_up, ctx.alloc((T, I)), epilogue=s.activation)
         else:
             up = linear(ctx, x, self.w_up, ctx.alloc((T, I)))
