@@ -1,9 +1,13 @@
-"""Kernels that Bumolix added to, each alone against a few lines of NumPy: the square of relu as
-the epilogue of the matrix-core product at every number of rows that picks another kernel of it,
-and the matrix-core attention with a chunk mask, the sink of score 0 and weights in two halves,
-against the plain softmax over the same cached keys."""
+"""Kernels that Bumolix added or added to, each alone against the plain function of the same
+mechanism or a few lines of NumPy: the square of relu as the epilogue of the matrix-core product
+at every number of rows that picks another kernel of it; the matrix-core attention with a chunk
+mask, the sink of score 0 and weights in two halves, against the plain softmax over the same
+cached keys; the two recurrences over two steps of two requests whose states are carried in
+slots, walked plainly and in segments."""
 import numpy as np
 import pytest
+
+from plain import bumolix_plain as P
 
 pytestmark = pytest.mark.gpu
 
@@ -119,3 +123,109 @@ def test_matrix_core_attention_with_chunks_and_the_sink(D, H, G, bs, chunk, sink
     got = rt.download_f32(out).reshape(T, H, D)
     err = np.abs(got - want).max(axis=(1, 2))
     assert err.max() < (0.012 if wide else 0.03), (int(np.argmax(err)), float(err.max()))
+
+
+def up32(rt, a):
+    _alive.append(rt.upload(np.ascontiguousarray(a, np.float32)))
+    return _alive[-1]
+
+
+STEPS = ([150, 37], [70, 1], [1, 129])       # tokens of requests 0 and 1 in three steps
+
+
+@pytest.mark.parametrize("seg", [0, 16, 64])
+@pytest.mark.parametrize("H,D,E", [(3, 12, 40), (2, 64, 128), (1, 200, 24), (2, 32, 8)])
+def test_gated_linear_attention_walk(H, D, E, seg):
+    """decayed_outer_products, the unit RMS with its gain and the gate, against zk_gla in 32-bit."""
+    from zse_amd.runtime.device import Runtime
+    rt = Runtime.get()
+    k = rt.kernels("float32")
+    rng = np.random.default_rng(H * 1000 + D + seg)
+    tau, eps, offset, slot_words = 3.0, 1e-5, 24, 24 + H * D * E + 8
+    total = [sum(st[r] for st in STEPS) for r in range(2)]
+    data = []
+    for r in range(2):
+        n = total[r]
+        q, kk = rng.normal(size=(n, H, D)), rng.normal(size=(n, H, D))
+        v, g, z = rng.normal(size=(n, H, E)), rng.normal(size=(n, H, E)), rng.normal(0.0, 2.0, (n, H, D))
+        data.append((q, kk, v, g, z))
+    bias, gain = rng.normal(1.5, 1.5, (H, D)), 1.0 + rng.normal(0, 0.3, E)
+    want = []
+    for q, kk, v, g, z in data:
+        alpha = np.exp(P.log_sigmoid(z + bias) / tau)
+        o = P.decayed_outer_products(q * D ** -0.5, kk, v, alpha, np.float64)
+        want.append(P.unit_rms(o, eps, np.float64) * gain * P.silu(g))
+    state = rt.zeros((2, slot_words), "float32")
+    slots = i32(rt, [1, 0])
+    done = [0, 0]
+    for st in STEPS:
+        T = sum(st)
+        rows = np.concatenate([np.concatenate([d[i][done[r]:done[r] + st[r]].reshape(st[r], -1) for i in range(4)], axis=1)
+                               for r, d in enumerate(data)])                      # q | k | v | g
+        z = np.concatenate([d[4][done[r]:done[r] + st[r]].reshape(st[r], -1) for r, d in enumerate(data)])
+        ld = 2 * H * D + 2 * H * E
+        X, Z = up32(rt, rows), up32(rt, z)
+        out, raw = rt.zeros((T, H * E), "float32"), rt.zeros((T, H * E), "float32")
+        max_q = -(-max(st) // 32) * 32 if max(st) > 1 else 1
+        nseg = 2 * -(-max_q // seg) if seg else 1
+        ss, sd = rt.zeros((nseg, H * D * E), "float32"), rt.zeros((nseg, H * D), "float32")
+        _alive.extend([out, raw, ss, sd])
+        k.zk_gla(X.ptr, ld, H * D, 2 * H * D, X.ptr + (2 * H * D + H * E) * 4, ld, Z.ptr, H * D, up32(rt, bias).ptr, tau,
+                 up32(rt, gain).ptr, state.ptr, slot_words, offset, i32(rt, [0, st[0], T]).ptr, slots.ptr,
+                 i32(rt, np.zeros(T)).ptr, out.ptr, raw.ptr, T, 2, max_q, H, D, E, eps, seg, ss.ptr if seg else None,
+                 sd.ptr if seg else None, rt.stream)
+        got = rt.download(out).reshape(T, H, E)
+        at = 0
+        for r in range(2):
+            ref = want[r][done[r]:done[r] + st[r]]
+            assert np.abs(got[at:at + st[r]] - ref).max() < 2e-4 * max(1.0, np.abs(ref).max()), (st, r)
+            at += st[r]
+            done[r] += st[r]
+    words = rt.download(state)
+    assert not words[:, :offset].any() and not words[:, offset + H * D * E:].any()     # nothing beside the state is touched
+
+
+@pytest.mark.parametrize("seg", [0, 16, 64])
+@pytest.mark.parametrize("I,N", [(72, 5), (200, 16), (64, 40), (9, 1)])
+def test_selective_scan_walk(I, N, seg):
+    """selective_scan and the gate against zk_selective_scan in 32-bit."""
+    from zse_amd.runtime.device import Runtime
+    rt = Runtime.get()
+    k = rt.kernels("float32")
+    rng = np.random.default_rng(I + N + seg)
+    offset, slot_words = 8, 8 + I * N + 4
+    total = [sum(st[r] for st in STEPS) for r in range(2)]
+    A_log, Dv, dt_bias = rng.normal(-1.0, 1.5, (I, N)), rng.normal(size=I), rng.normal(-1.0, 1.0, I)
+    data, want = [], []
+    for r in range(2):
+        n = total[r]
+        u, dt, z = rng.normal(size=(n, I)), rng.normal(0, 1.5, (n, I)), rng.normal(size=(n, I))
+        B, C = rng.normal(size=(n, N)), rng.normal(size=(n, N))
+        data.append((u, dt, z, B, C))
+        y = P.selective_scan(u, P.softplus(dt + dt_bias), -np.exp(A_log), B, C, Dv, np.float64)
+        want.append(y * P.silu(z))
+    state = rt.zeros((2, slot_words), "float32")
+    slots = i32(rt, [1, 0])
+    done = [0, 0]
+    for st in STEPS:
+        T = sum(st)
+        cut = lambda i: np.concatenate([d[i][done[r]:done[r] + st[r]] for r, d in enumerate(data)])
+        bc = np.concatenate([np.zeros((T, 3)), cut(3), cut(4)], axis=1)            # three columns of something else first
+        out = rt.zeros((T, I), "float32")
+        max_q = -(-max(st) // 32) * 32 if max(st) > 1 else 1
+        nseg = 2 * -(-max_q // seg) if seg else 1
+        ss, sd = rt.zeros((nseg, I * N), "float32"), rt.zeros((nseg, I), "float32")
+        _alive.extend([out, ss, sd])
+        k.zk_selective_scan(up32(rt, cut(0)).ptr, I, up32(rt, cut(1)).ptr, I, up32(rt, dt_bias).ptr, up32(rt, bc).ptr, 3 + 2 * N,
+                            3, 3 + N, up32(rt, A_log).ptr, up32(rt, Dv).ptr, up32(rt, cut(2)).ptr, I, state.ptr, slot_words,
+                            offset, i32(rt, [0, st[0], T]).ptr, slots.ptr, out.ptr, T, 2, I, N, max_q, seg,
+                            ss.ptr if seg else None, sd.ptr if seg else None, rt.stream)
+        got = rt.download(out)
+        at = 0
+        for r in range(2):
+            ref = want[r][done[r]:done[r] + st[r]]
+            assert np.abs(got[at:at + st[r]] - ref).max() < 2e-4 * max(1.0, np.abs(ref).max()), (st, r)
+            at += st[r]
+            done[r] += st[r]
+    words = rt.download(state)
+    assert not words[:, :offset].any() and not words[:, offset + I * N:].any()
