@@ -73,7 +73,8 @@ def plain_attention(q, kk, v, pos0, scale, chunk, sink):
 
 @pytest.mark.parametrize("wide", [0, 1])
 @pytest.mark.parametrize("D,H,G,bs,chunk,sink", [(16, 4, 2, 4, 24, 1), (64, 2, 1, 16, 100, 1), (128, 8, 2, 16, 700, 1),
-                                                 (32, 3, 3, 8, 0, 1), (128, 4, 4, 16, 64, 0)])
+                                                 (32, 3, 3, 8, 0, 1), (128, 4, 4, 16, 64, 0), (64, 4, 1, 16, 1, 1),
+                                                 (32, 4, 2, 8, 33, 1), (256, 2, 2, 32, 1000, 1)])
 def test_matrix_core_attention_with_chunks_and_the_sink(D, H, G, bs, chunk, sink, wide):
     """Three requests of one step: a long portion from position 0 (one request, few heads: its keys are
     cut into ranges), a portion that begins inside a chunk behind a cached context, and a single
