@@ -67,6 +67,10 @@ class RotarySpec:
     # ramp over the pair numbers in between; sines and cosines are multiplied by 0.1 ln(factor) + 1
     scaling: Optional[Tuple[float, float, float, float]] = None
     linear_factor: Optional[float] = None   # every frequency is divided by it (positions stretched); magnitudes stay 1
+    # (factor, low, high, original): each frequency f judged by its wavelength l = 2 pi / f: it stays where
+    # l < original / high, is divided by ``factor`` where l > original / low, and in between becomes
+    # (1 - s) f / factor + s f with s = (original / l - low) / (high - low); magnitudes stay 1
+    wavelength_scaling: Optional[Tuple[float, float, float, float]] = None
 
 
 @dataclass(frozen=True)
@@ -104,6 +108,11 @@ class AttentionSpec:
     gate: Optional[str] = None               # [num_heads * value_dim, hidden]: heads times sigmoid(W_g x) before W_o
     wide_weights: bool = False               # the softmax's weights are not rounded to 8 bits of mantissa before they
     #                                          meet the values (the matrix-core kernel sends them in two halves)
+    q_row_norm: Optional[str] = None         # gain [num_heads * head_dim] of an RMS norm over a token's whole query row
+    #                                          (all heads at once, after the bias, before rotation; eps is norm_eps)
+    k_row_norm: Optional[str] = None         # the same over the whole key row, gain [num_kv_heads * head_dim]
+    values_are_keys: bool = False            # no value projection: a value is its key as projected (with its bias,
+    #                                          before norm and rotation); ``names`` and ``biases`` hold no role v
 
 
 @dataclass(frozen=True)
@@ -122,9 +131,39 @@ class LatentAttentionSpec:
     scale: float
     eps: float                       # of the latent's norm
     position: Any                    # a rotary spec over rotary_dim channels
-    names: Dict[str, str]            # roles q, down, down_norm, up_k, up_v, o, sinks (optional)
+    names: Dict[str, str]            # roles q, down, down_norm, up_k, up_v, o, sinks (optional),
+    #                                  q_down, q_down_norm, gate (optional, below)
     window: Optional[int] = None
     kind: str = "latent_attention"
+    # queries through a latent of their own: c_q = rms_norm(W_q_down x) * gain (eps as above), q = W_q c_q;
+    # ``names["q"]`` is then [heads * (head_dim + rotary_dim), query_latent_dim]
+    query_latent_dim: Optional[int] = None
+    # names["gate"]: [num_heads, hidden]; head h's output times sigmoid(W_gate x)_h, one number a head
+
+
+@dataclass(frozen=True)
+class DifferentialAttentionSpec:
+    """Two softmax maps per head over the same values, combined as a difference.  A query head's
+    row is [map 1 | map 2] of ``head_dim`` each, a key head's likewise; a value head has
+    ``value_dim``.  No rotation.  Queries are multiplied by a temperature of their position,
+    1 + temp_coef ln(floor((p + 1) / temp_every) + 1) (``temp_every`` 0: none); scores
+    (q . k) scale, then cap tanh(s / cap); with lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff the
+    head's result is o = a1 - lambda a2, divided by its root mean square (eps, no gain), times
+    (1 - diff)."""
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int                    # of one map
+    value_dim: int
+    scale: float
+    softcap: Optional[float]
+    window: Optional[int]
+    diff: float
+    eps: float
+    temp_coef: float
+    temp_every: int
+    names: Dict[str, str]            # roles q, k, v, o, lq1, lk1, lq2, lk2
+    kind: str = "differential_attention"
 
 
 @dataclass(frozen=True)
@@ -241,6 +280,8 @@ class RoutedMLPSpec:
     shared: Any = None               # a GatedMLPSpec or None
     scale_input: bool = True
     kind: str = "routed_mlp"
+    scoring: str = "sigmoid"         # or "softmax": scores exp(z) / sum over all experts
+    shared_gate: Optional[str] = None   # [1, hidden]: the shared layer's result times sigmoid(W x), a number a token
 
 
 @dataclass(frozen=True)
@@ -280,6 +321,17 @@ class StreamsBlockSpec:
 
 
 @dataclass(frozen=True)
+class PairTableSpec:
+    """A table of token pairs whose row (previous token * mul_prev + token * mul_cur) mod buckets is
+    added to the embedded row; a sequence's first token takes row ``buckets`` (the table's last).
+    The previous token is part of a request's state."""
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+    weight: str                      # [buckets + 1, hidden]
+
+
+@dataclass(frozen=True)
 class EmbeddingSpec:
     vocab_size: int
     hidden_size: int
@@ -287,6 +339,7 @@ class EmbeddingSpec:
     weight: str
     kind: str = "embedding"
     copies: int = 1                  # the row is written this many times (one per residual stream)
+    pairs: Optional[PairTableSpec] = None
 
 
 @dataclass(frozen=True)

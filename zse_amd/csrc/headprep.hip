@@ -145,6 +145,115 @@ extern "C" int zk_head_prep(void* qkv, const int* positions, const int* slot_map
                           v_interleaved, kcache, vcache, T, nh, nkv, D, E, bs, v_transposed, nullptr, 1.0f, 0, stream);
 }
 
+// Queries and keys whose norm runs over the whole row of heads, and values that are the keys.
+//
+//   q <- rot_p( (q + bq) / sqrt(mean over all nh D channels + eps) * gq ),   gq of nh D numbers
+//   k <- rot_p( (k + bk) / sqrt(mean over all nkv D channels + eps) * gk )
+//   v  = k + bk as projected (before norm and rotation), where ``values_are_keys``
+//
+// One block per token: a row holds nh query heads, then nkv key heads of D (and, without
+// values_are_keys, nkv value heads of E that are stored as they are).  Float throughout, one
+// rounding at the store.  The block is 256 wide whatever the step, so a row's sums do not
+// depend on what else the step holds.
+__global__ __launch_bounds__(256) void row_prep_kernel(
+    act_t* __restrict__ qk, int ld, const int* __restrict__ positions, const int* __restrict__ slot_map,
+    const float* __restrict__ bias, const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
+    const float* __restrict__ inv_freq, int rot_dims, act_t* __restrict__ kcache, act_t* __restrict__ vcache, int nh,
+    int nkv, int D, int E, int bs, int v_transposed, int values_are_keys) {
+  extern __shared__ float row[];                 // [(nh + nkv) D]
+  __shared__ float red[17];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int pos = positions[t];
+  if (pos < 0) return;
+  const int nq = nh * D, nk = nkv * D;
+  act_t* src = qk + (size_t)t * ld;
+  float sq = 0.f, sk = 0.f;
+  for (int i = tid; i < nq + nk; i += 256) {
+    float x = to_f32(src[i]);
+    if (bias) x += bias[i];
+    row[i] = x;
+    if (i < nq) sq = fmaf(x, x, sq);
+    else sk = fmaf(x, x, sk);
+  }
+  sq = block_sum(sq, red);
+  sk = block_sum(sk, red);
+  const int slot = slot_map ? slot_map[t] : -1;
+  const size_t page = slot >= 0 ? slot / bs : 0, off = slot >= 0 ? slot % bs : 0;
+  if (slot >= 0) {
+    // the values: the keys before norm and rotation, or the row's own value heads
+    const int nv = nkv * E;
+    for (int i = tid; i < nv; i += 256) {
+      const int g = i / E, d = i % E;
+      float x;
+      if (values_are_keys) x = row[nq + i];
+      else {
+        x = to_f32(src[nq + nk + i]);
+        if (bias) x += bias[nq + nk + i];
+      }
+      if (v_transposed) vcache[(page * nkv + g) * (size_t)E * bs + (size_t)d * bs + off] = from_f32<act_t>(x);
+      else vcache[((page * nkv + g) * bs + off) * E + d] = from_f32<act_t>(x);
+    }
+  }
+  __syncthreads();
+  if (q_gain) {
+    const float inv = 1.0f / sqrtf(sq / (float)nq + eps);
+    for (int i = tid; i < nq; i += 256) row[i] = row[i] * inv * q_gain[i];
+  }
+  if (k_gain) {
+    const float inv = 1.0f / sqrtf(sk / (float)nk + eps);
+    for (int i = tid; i < nk; i += 256) row[nq + i] = row[nq + i] * inv * k_gain[i];
+  }
+  __syncthreads();
+  if (inv_freq) {
+    const int half = rot_dims / 2;
+    for (int i = tid; i < (nh + nkv) * half; i += 256) {
+      const int head = i / half, m = i % half;
+      float sn, cs, ra, rb;
+      sincosf((float)pos * inv_freq[m], &sn, &cs);
+      float* hp = row + head * D;
+      rotate_pair(hp[m], hp[m + half], sn, cs, ra, rb);
+      hp[m] = ra;
+      hp[m + half] = rb;
+    }
+    __syncthreads();
+  }
+  for (int i = tid; i < nq; i += 256) src[i] = from_f32<act_t>(row[i]);
+  if (slot >= 0)
+    for (int i = tid; i < nk; i += 256) {
+      const int g = i / D, d = i % D;
+      kcache[((page * nkv + g) * bs + off) * D + d] = from_f32<act_t>(row[nq + i]);
+    }
+}
+
+// qk: [T, ld], changed in place (the queries) and stored (keys, values).  bias (may be null): one
+// float per channel of a row.  q_gain [nh D], k_gain [nkv D] (either may be null: no norm).
+// values_are_keys: E == D and a row holds no value heads.
+extern "C" int zk_row_prep(void* qk, int ld, const int* positions, const int* slot_map, const float* bias,
+                           const float* q_gain, const float* k_gain, float eps, const float* inv_freq, int rot_dims,
+                           void* kcache, void* vcache, int T, int nh, int nkv, int D, int E, int bs, int v_transposed,
+                           int values_are_keys, void* stream) {
+  ZK_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && D > 0 && E > 0 && bs > 0, "zk_row_prep: bad sizes");
+  ZK_REQUIRE(!values_are_keys || E == D, "zk_row_prep: values that are keys have the keys' size");
+  ZK_REQUIRE(ld >= (nh + nkv) * D + (values_are_keys ? 0 : nkv * E), "zk_row_prep: rows shorter than their heads");
+  ZK_REQUIRE(inv_freq == nullptr || (rot_dims % 2 == 0 && rot_dims > 0 && rot_dims <= D),
+             "zk_row_prep: the rotated channels must be even in number and at most the head's");
+  ZK_REQUIRE(kcache != nullptr && vcache != nullptr && slot_map != nullptr, "zk_row_prep: no cache to store into");
+  const size_t lds = (size_t)(nh + nkv) * D * sizeof(float);
+  ZK_REQUIRE(lds <= 64 * 1024, "zk_row_prep: rows of more than 16384 channels are not supported");
+  if (T == 0) return 0;
+  static bool raised = false;
+  if (!raised) {
+    hipFuncSetAttribute((const void*)row_prep_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    raised = true;
+  }
+  row_prep_kernel<<<T, 256, lds, (hipStream_t)stream>>>((act_t*)qk, ld, positions, slot_map, bias, q_gain, k_gain, eps,
+                                                       inv_freq, rot_dims, (act_t*)kcache, (act_t*)vcache, nh, nkv, D, E,
+                                                       bs, v_transposed, values_are_keys);
+  return zk_launch_status("zk_row_prep");
+}
+
+static const int row_prep_entered =
+    zk_steplist_register("zk_row_prep", zk_packed::Call<zk_row_prep>::nargs, (void*)zk_packed::Call<zk_row_prep>::call);
 static const int head_prep_entered =
     zk_steplist_register("zk_head_prep", zk_packed::Call<zk_head_prep>::nargs, (void*)zk_packed::Call<zk_head_prep>::call);
 static const int head_prep_unit_entered = zk_steplist_register(

@@ -18,9 +18,10 @@ extern "C" int zk_steplist_register(const char* name, int nargs, void* fn);
 // qa[t, head, C:].  The latent (blockIdx.y == H): the normed c and the rotated key part go to
 // the cache row of the token's slot.
 __global__ __launch_bounds__(256) void latent_prep_kernel(
-    const act_t* __restrict__ qd, int ld, const int* __restrict__ positions, const int* __restrict__ slot_map,
-    const float* __restrict__ gain, float eps, const float* __restrict__ freq, float rot_scale, int interleaved,
-    act_t* __restrict__ qa, act_t* __restrict__ kcache, int H, int D, int R, int C, int bs) {
+    const act_t* __restrict__ qd, int ld, const act_t* __restrict__ down, int ldd, const int* __restrict__ positions,
+    const int* __restrict__ slot_map, const float* __restrict__ gain, float eps, const float* __restrict__ freq,
+    float rot_scale, int interleaved, act_t* __restrict__ qa, act_t* __restrict__ kcache, int H, int D, int R, int C,
+    int bs) {
   __shared__ float red[17];
   const int t = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
   const int pos = positions[t];
@@ -43,7 +44,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
   }
   const int slot = slot_map[t];
   if (slot < 0) return;
-  const act_t* src = qd + (size_t)t * ld + (size_t)H * (D + R);
+  const act_t* src = down + (size_t)t * ldd;
   act_t* dst = kcache + (size_t)slot * (C + R);           // one key head: row (page * bs + offset)
   float ss = 0.f;
   for (int i = tid; i < C; i += 256) {
@@ -142,17 +143,28 @@ extern "C" {
 
 // qd: [T, ld]: H query heads of D + R, then C + R of the down-projection.  qa: [T, H, C + R], of
 // which this writes [.., C:].  kcache: [pages, 1, bs, C + R].  freq: float [R / 2].
-int zk_latent_prep(const void* qd, int ld, const int* positions, const int* slot_map, const float* gain, float eps,
-                   const float* freq, float rot_scale, int interleaved, void* qa, void* kcache, int T, int H, int D,
-                   int R, int C, int bs, void* stream) {
+// q: [T, ldq], H query heads of D + R; down: [T, ldd], C + R of the down-projection, wherever the
+// two lie.
+int zk_latent_prep_ext(const void* q, int ldq, const void* down, int ldd, const int* positions, const int* slot_map,
+                       const float* gain, float eps, const float* freq, float rot_scale, int interleaved, void* qa,
+                       void* kcache, int T, int H, int D, int R, int C, int bs, void* stream) {
   ZK_REQUIRE(T >= 0 && H > 0 && D > 0 && R >= 0 && R % 2 == 0 && C > 0 && bs > 0, "zk_latent_prep: bad sizes");
-  ZK_REQUIRE(ld >= H * (D + R) + C + R, "zk_latent_prep: rows too short");
+  ZK_REQUIRE(ldq >= H * (D + R) && ldd >= C + R, "zk_latent_prep: rows too short");
   ZK_REQUIRE(H < 65535 && (R == 0 || freq != nullptr), "zk_latent_prep: too many heads, or no frequencies");
   if (T == 0) return 0;
   dim3 grid(T, H + 1);
-  latent_prep_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)qd, ld, positions, slot_map, gain, eps, freq,
-                                                            rot_scale, interleaved, (act_t*)qa, (act_t*)kcache, H, D, R, C, bs);
+  latent_prep_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)q, ldq, (const act_t*)down, ldd, positions, slot_map,
+                                                            gain, eps, freq, rot_scale, interleaved, (act_t*)qa,
+                                                            (act_t*)kcache, H, D, R, C, bs);
   return zk_launch_status("zk_latent_prep");
+}
+
+int zk_latent_prep(const void* qd, int ld, const int* positions, const int* slot_map, const float* gain, float eps,
+                   const float* freq, float rot_scale, int interleaved, void* qa, void* kcache, int T, int H, int D,
+                   int R, int C, int bs, void* stream) {
+  ZK_REQUIRE(H > 0 && D > 0 && R >= 0 && C > 0 && ld >= H * (D + R) + C + R, "zk_latent_prep: rows too short");
+  return zk_latent_prep_ext(qd, ld, (const act_t*)qd + (size_t)H * (D + R), ld, positions, slot_map, gain, eps, freq,
+                            rot_scale, interleaved, qa, kcache, T, H, D, R, C, bs, stream);
 }
 
 // x: head h of token t at x[t * ldx + h * x_head], K channels; out likewise with ldo, o_head, N.
@@ -185,6 +197,7 @@ int zk_heads_linear(const void* x, int ldx, int x_head, const void* w, int w_kn,
 }  // extern "C"
 
 ZK_ENTER(zk_latent_prep)
+ZK_ENTER(zk_latent_prep_ext)
 ZK_ENTER(zk_heads_linear)
 
 #if ZSE_ACT_BF16

@@ -5,6 +5,11 @@
 //   g = min(Wg x', limit),  u = clamp(Wu x', -limit, limit),  y = g sigmoid(1.702 g) (u + 1)
 //   out_t = sum over the chosen experts, in the order they were chosen, of Wd y
 //
+// Variants, as parameters of the ``_ext`` entry points: scores softmax(router logits) over all experts
+// instead of sigmoids; the weight on the expert's output instead of its input (out_t = sum s_e Wd y);
+// y = silu(g) u instead of the clamped form.  ``zk_gate_rows`` multiplies float rows by the sigmoid
+// of a number a row (a shared layer's gate).
+//
 // Two ways through the experts.  Few tokens (decoding): one block per (token, choice) multiplies
 // the expert's rows by the token's row, and the weights stream once per choice.  Many tokens
 // (bfloat16 only): the (token, choice) pairs are sorted by expert on the device, the scaled rows
@@ -28,15 +33,41 @@ __device__ __forceinline__ float clamped_swiglu(float g, float u, float limit) {
   return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
 }
 
+__device__ __forceinline__ float expert_act(float g, float u, float limit, int act) {
+  return act == 1 ? g / (1.0f + expf(-g)) * u : clamped_swiglu(g, u, limit);
+}
+
 // ---- the router: one wave per token
-__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, int E, int top,
-                                                       int* __restrict__ ids, float* __restrict__ wts) {
+__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, int ld, int E, int top,
+                                                       int* __restrict__ ids, float* __restrict__ wts, int softmax) {
   const int t = blockIdx.x, lane = threadIdx.x;
   float s[MOE_MAX_EXPERTS / 64];
+  if (softmax) {
+    // scores exp(z - max) / sum over all experts, in float
+    float mx = -INFINITY;
 #pragma unroll
-  for (int i = 0; i < MOE_MAX_EXPERTS / 64; i++) {
-    const int e = lane + 64 * i;
-    s[i] = e < E ? 1.0f / (1.0f + expf(-logits[(size_t)t * E + e])) : -1.f;
+    for (int i = 0; i < MOE_MAX_EXPERTS / 64; i++) {
+      const int e = lane + 64 * i;
+      s[i] = e < E ? logits[(size_t)t * ld + e] : -INFINITY;
+      mx = fmaxf(mx, s[i]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_EXPERTS / 64; i++) {
+      const int e = lane + 64 * i;
+      s[i] = e < E ? expf(s[i] - mx) : 0.f;
+      sum += s[i];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_EXPERTS / 64; i++) s[i] = (lane + 64 * i) < E ? s[i] / sum : -1.f;
+  } else {
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_EXPERTS / 64; i++) {
+      const int e = lane + 64 * i;
+      s[i] = e < E ? 1.0f / (1.0f + expf(-logits[(size_t)t * ld + e])) : -1.f;
+    }
   }
   for (int k = 0; k < top; k++) {
     float best = -2.f;
@@ -112,14 +143,14 @@ __device__ __forceinline__ float row_dot(const act_t* __restrict__ w, const floa
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(const act_t* __restrict__ x, const int* __restrict__ ids,
                                                           const float* __restrict__ wts, const act_t* __restrict__ w_gu,
                                                           act_t* __restrict__ y, int top, int W, int F, float limit,
-                                                          int rows_per_block) {
+                                                          int rows_per_block, int act, int on_out) {
   extern __shared__ float xs[];                   // [W]
   const int pair = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int e = ids[pair];
   const float s = wts[pair];
   const int t = pair / top;
   const act_t* xr = x + (size_t)t * W;
-  for (int i = tid; i < W; i += 256) xs[i] = to_f32(from_f32<act_t>(s * to_f32(xr[i])));
+  for (int i = tid; i < W; i += 256) xs[i] = on_out ? to_f32(xr[i]) : to_f32(from_f32<act_t>(s * to_f32(xr[i])));
   __syncthreads();
   const act_t* wg = w_gu + (size_t)e * 2 * F * W;
   const int n0 = blockIdx.y * rows_per_block;
@@ -127,14 +158,15 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const act_t* __restric
     const act_t* gr = wg + (size_t)n * W;
     const act_t* ur = wg + (size_t)(F + n) * W;
     const float g = row_dot(gr, xs, W, lane), u = row_dot(ur, xs, W, lane);
-    if (lane == 0) y[(size_t)pair * F + n] = from_f32<act_t>(clamped_swiglu(g, u, limit));
+    if (lane == 0) y[(size_t)pair * F + n] = from_f32<act_t>(expert_act(g, u, limit, act));
   }
 }
 
 // out[t, n] = sum_k Wd[e_k][n] . y[(t, k)]
 __global__ __launch_bounds__(256) void moe_down_kernel(const act_t* __restrict__ y, const int* __restrict__ ids,
                                                        const act_t* __restrict__ w_down, float* __restrict__ out,
-                                                       int top, int W, int F, int rows_per_block) {
+                                                       int top, int W, int F, int rows_per_block,
+                                                       const float* __restrict__ wts) {
   extern __shared__ float ys[];                   // [top][F]
   const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int i = tid; i < top * F; i += 256) ys[i] = to_f32(y[(size_t)t * top * F + i]);
@@ -144,7 +176,8 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const act_t* __restrict__
     float total = 0.f;
     for (int k = 0; k < top; k++) {
       const act_t* wr = w_down + ((size_t)ids[(size_t)t * top + k] * W + n) * F;
-      total += row_dot(wr, ys + k * F, F, lane);
+      const float d = row_dot(wr, ys + k * F, F, lane);
+      total += wts ? wts[(size_t)t * top + k] * d : d;
     }
     if (lane == 0) out[(size_t)t * W + n] = total;
   }
@@ -186,7 +219,7 @@ __global__ void moe_gather_kernel(const act_t* __restrict__ x, const int* __rest
                                   const float* __restrict__ wts, act_t* __restrict__ xg, int top, int W) {
   const int i = blockIdx.x;
   const int pair = order[i];
-  const float s = wts[pair];
+  const float s = wts ? wts[pair] : 1.0f;
   const act_t* xr = x + (size_t)(pair / top) * W;
   for (int c = threadIdx.x; c < W; c += blockDim.x) xg[(size_t)i * W + c] = from_f32<act_t>(s * to_f32(xr[c]));
 }
@@ -210,7 +243,7 @@ template <int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                           const int* __restrict__ first, int E, int N, int K,
                                                           __bf16* __restrict__ y, float* __restrict__ out_rows,
-                                                          float limit) {
+                                                          float limit, int act) {
   __shared__ __bf16 As[GG_TM][GG_TK + GG_PAD];
   __shared__ __bf16 Bs[(MODE == 0 ? 2 : 1) * GG_TN][GG_TK + GG_PAD];
   __shared__ int tile_e, tile_row, tile_end;
@@ -270,7 +303,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const __bf16* __restri
   for (int i = 0; i < 16; i++) {
     const int r = wm + (i / 4) * 8 + (lane >> 5) * 4 + (i % 4);
     if (r < rows && col < N) {
-      if (MODE == 0) y[(size_t)(row0 + r) * N + col] = (__bf16)clamped_swiglu(acc0[i], acc1[i], limit);
+      if (MODE == 0) y[(size_t)(row0 + r) * N + col] = (__bf16)expert_act(acc0[i], acc1[i], limit, act);
       else out_rows[(size_t)(row0 + r) * N + col] = acc0[i];
     }
   }
@@ -278,11 +311,14 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const __bf16* __restri
 
 // out[t, :] = sum over t's choices, in their order, of the sorted rows' results
 __global__ void moe_combine_kernel(const float* __restrict__ rows, const int* __restrict__ place, float* __restrict__ out,
-                                   int top, int W) {
+                                   int top, int W, const float* __restrict__ wts) {
   const int t = blockIdx.x;
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float total = 0.f;
-    for (int k = 0; k < top; k++) total += rows[(size_t)place[(size_t)t * top + k] * W + c];
+    for (int k = 0; k < top; k++) {
+      const float v = rows[(size_t)place[(size_t)t * top + k] * W + c];
+      total += wts ? wts[(size_t)t * top + k] * v : v;
+    }
     out[(size_t)t * W + c] = total;
   }
 }
@@ -293,23 +329,45 @@ __global__ void moe_place_kernel(const int* __restrict__ order, int* __restrict_
 }
 #endif
 
+// rows[t, :] *= sigmoid(z[t * ld])
+__global__ void gate_rows_kernel(float* __restrict__ rows, const float* __restrict__ z, int ld, int W) {
+  const int t = blockIdx.x;
+  const float g = 1.0f / (1.0f + expf(-z[(size_t)t * ld]));
+  for (int c = threadIdx.x; c < W; c += blockDim.x) rows[(size_t)t * W + c] *= g;
+}
+
 extern "C" {
 
 // logits: float [T, E] -> ids int32 [T, top], wts float [T, top] (the scores themselves).
 // (device memory that a kernel writes is passed as void*: an ``int*`` argument means a result the
 // host reads, which a launch list replaces)
-int zk_moe_route(const float* logits, void* ids, float* wts, int T, int E, int top, void* stream) {
-  ZK_REQUIRE(T >= 0 && E > 0 && top > 0 && top <= E, "zk_moe_route: bad sizes");
+// ld: the distance between rows of logits (>= E; a row may hold more than the experts' logits).
+// softmax: the scores are exp(z) / sum over all experts instead of sigmoid(z).
+int zk_moe_route_ext(const float* logits, int ld, void* ids, float* wts, int T, int E, int top, int softmax, void* stream) {
+  ZK_REQUIRE(T >= 0 && E > 0 && top > 0 && top <= E && ld >= E, "zk_moe_route: bad sizes");
   ZK_REQUIRE(E <= MOE_MAX_EXPERTS && top <= MOE_MAX_TOP, "zk_moe_route: up to 1024 experts and 16 choices");
   if (T == 0) return 0;
-  moe_route_kernel<<<T, 64, 0, (hipStream_t)stream>>>(logits, E, top, (int*)ids, wts);
+  moe_route_kernel<<<T, 64, 0, (hipStream_t)stream>>>(logits, ld, E, top, (int*)ids, wts, softmax);
   return zk_launch_status("zk_moe_route");
+}
+
+int zk_moe_route(const float* logits, void* ids, float* wts, int T, int E, int top, void* stream) {
+  return zk_moe_route_ext(logits, E, ids, wts, T, E, top, 0, stream);
+}
+
+// rows: float [T, W], each multiplied by sigmoid(z[t * ld]).
+int zk_gate_rows(float* rows, const float* z, int ld, int T, int W, void* stream) {
+  ZK_REQUIRE(T >= 0 && W > 0 && ld > 0 && rows != nullptr && z != nullptr, "zk_gate_rows: bad arguments");
+  if (T == 0) return 0;
+  gate_rows_kernel<<<T, 256, 0, (hipStream_t)stream>>>(rows, z, ld, W);
+  return zk_launch_status("zk_gate_rows");
 }
 
 // x: [T, W]; w_gu: [E][2F][W], an expert's gate rows, then its up rows; w_down: [E][W][F].
 // y: scratch [T * top, F] activations; out: float [T, W].
-int zk_moe_experts(const void* x, const int* ids, const float* wts, const void* w_gu, const void* w_down, void* y,
-                   float* out, int T, int top, int W, int F, float limit, void* stream) {
+// act: 0 the clamped form, 1 silu(gate) up.  on_out: the weight multiplies the expert's output.
+int zk_moe_experts_ext(const void* x, const int* ids, const float* wts, const void* w_gu, const void* w_down, void* y,
+                       float* out, int T, int top, int W, int F, float limit, int act, int on_out, void* stream) {
   ZK_REQUIRE(T >= 0 && top > 0 && top <= MOE_MAX_TOP && W > 0 && F > 0, "zk_moe_experts: bad sizes");
   ZK_REQUIRE(T <= 65535 && (size_t)T * top <= 0x7fffffff, "zk_moe_experts: more than 65535 rows");
   ZK_REQUIRE((size_t)W * 4 <= 64 * 1024 && (size_t)top * F * 4 <= 64 * 1024, "zk_moe_experts: rows too wide for local memory");
@@ -323,11 +381,16 @@ int zk_moe_experts(const void* x, const int* ids, const float* wts, const void* 
   }
   dim3 grid_up(T * top, (F + rpb - 1) / rpb);
   moe_gate_up_kernel<<<grid_up, 256, (size_t)W * 4, (hipStream_t)stream>>>((const act_t*)x, ids, wts, (const act_t*)w_gu,
-                                                                          (act_t*)y, top, W, F, limit, rpb);
+                                                                          (act_t*)y, top, W, F, limit, rpb, act, on_out);
   dim3 grid(T, (W + rpb - 1) / rpb);
   moe_down_kernel<<<grid, 256, (size_t)top * F * 4, (hipStream_t)stream>>>((const act_t*)y, ids, (const act_t*)w_down, out, top,
-                                                                         W, F, rpb);
+                                                                         W, F, rpb, on_out ? wts : nullptr);
   return zk_launch_status("zk_moe_experts");
+}
+
+int zk_moe_experts(const void* x, const int* ids, const float* wts, const void* w_gu, const void* w_down, void* y,
+                   float* out, int T, int top, int W, int F, float limit, void* stream) {
+  return zk_moe_experts_ext(x, ids, wts, w_gu, w_down, y, out, T, top, W, F, limit, 0, 0, stream);
 }
 
 // gu: [T, 2F] -> y [T, F]
@@ -342,9 +405,9 @@ int zk_clamped_glu(const void* gu, void* y, int T, int F, float limit, void* str
 #if ZSE_ACT_BF16
 // The same through the grouped matrix-core product.  work: int32 [E + 1 + 2 * T * top] (first,
 // order, place); xg: [T * top, W] and y: [T * top, F] bfloat16; rows: float [T * top, W].
-int zk_moe_experts_grouped(const void* x, const int* ids, const float* wts, const void* w_gu, const void* w_down,
-                           void* work, void* xg, void* y, float* rows, float* out, int T, int E, int top, int W, int F,
-                           float limit, void* stream) {
+int zk_moe_experts_grouped_ext(const void* x, const int* ids, const float* wts, const void* w_gu, const void* w_down,
+                               void* work, void* xg, void* y, float* rows, float* out, int T, int E, int top, int W, int F,
+                               float limit, int act, int on_out, void* stream) {
   ZK_REQUIRE(T >= 0 && top > 0 && top <= MOE_MAX_TOP && W > 0 && F > 0 && E > 0 && E <= MOE_MAX_EXPERTS,
              "zk_moe_experts_grouped: bad sizes");
   ZK_REQUIRE(W % 8 == 0 && F % 8 == 0, "zk_moe_experts_grouped: widths in whole groups of eight");
@@ -357,14 +420,20 @@ int zk_moe_experts_grouped(const void* x, const int* ids, const float* wts, cons
   hipStream_t st = (hipStream_t)stream;
   moe_sort_kernel<<<1, 1024, 0, st>>>(ids, pairs, E, first, order);
   moe_place_kernel<<<(pairs + 255) / 256, 256, 0, st>>>(order, place, pairs);
-  moe_gather_kernel<<<pairs, 256, 0, st>>>((const act_t*)x, order, wts, (act_t*)xg, top, W);
+  moe_gather_kernel<<<pairs, 256, 0, st>>>((const act_t*)x, order, on_out ? nullptr : wts, (act_t*)xg, top, W);
   const int tiles = (pairs + GG_TM - 1) / GG_TM + E;        // each expert may end in a tile that is not full
   dim3 g0(tiles, (F + GG_TN - 1) / GG_TN);
-  moe_grouped_kernel<0><<<g0, 256, 0, st>>>((const __bf16*)xg, (const __bf16*)w_gu, first, E, F, W, (__bf16*)y, nullptr, limit);
+  moe_grouped_kernel<0><<<g0, 256, 0, st>>>((const __bf16*)xg, (const __bf16*)w_gu, first, E, F, W, (__bf16*)y, nullptr, limit, act);
   dim3 g1(tiles, (W + GG_TN - 1) / GG_TN);
-  moe_grouped_kernel<1><<<g1, 256, 0, st>>>((const __bf16*)y, (const __bf16*)w_down, first, E, W, F, nullptr, rows, 0.f);
-  moe_combine_kernel<<<T, 256, 0, st>>>(rows, place, out, top, W);
+  moe_grouped_kernel<1><<<g1, 256, 0, st>>>((const __bf16*)y, (const __bf16*)w_down, first, E, W, F, nullptr, rows, 0.f, 0);
+  moe_combine_kernel<<<T, 256, 0, st>>>(rows, place, out, top, W, on_out ? wts : nullptr);
   return zk_launch_status("zk_moe_experts_grouped");
+}
+
+int zk_moe_experts_grouped(const void* x, const int* ids, const float* wts, const void* w_gu, const void* w_down,
+                           void* work, void* xg, void* y, float* rows, float* out, int T, int E, int top, int W, int F,
+                           float limit, void* stream) {
+  return zk_moe_experts_grouped_ext(x, ids, wts, w_gu, w_down, work, xg, y, rows, out, T, E, top, W, F, limit, 0, 0, stream);
 }
 #endif
 
@@ -372,7 +441,11 @@ int zk_moe_experts_grouped(const void* x, const int* ids, const float* wts, cons
 
 #if ZSE_ACT_BF16
 ZK_ENTER(zk_moe_experts_grouped)
+ZK_ENTER(zk_moe_experts_grouped_ext)
 #endif
+ZK_ENTER(zk_moe_route_ext)
+ZK_ENTER(zk_moe_experts_ext)
+ZK_ENTER(zk_gate_rows)
 ZK_ENTER(zk_moe_route)
 ZK_ENTER(zk_moe_experts)
 ZK_ENTER(zk_clamped_glu)

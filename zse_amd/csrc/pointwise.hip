@@ -1,7 +1,8 @@
 // Element by element: an activation without a gate, and a gate on the heads of a mixer.
 //
 //   zk_unary_act:   out = act(x)                        act 0: max(x, 0)^2
-//   zk_gate_heads:  o <- o * sigmoid(g)                 g read from rows of another width
+//   zk_gate_heads:  o <- o * sigmoid(g)                 g read from rows of another width; one g
+//                                                       for every ``per`` channels (a number a head)
 //
 // Arithmetic is float; one rounding to the activation type at the store.
 #include "common.h"
@@ -18,11 +19,11 @@ __global__ void unary_act_kernel(const act_t* __restrict__ x, act_t* __restrict_
   out[i] = from_f32<act_t>(v * v);
 }
 
-__global__ void gate_heads_kernel(act_t* __restrict__ o, const act_t* __restrict__ g, int ldg, int W) {
+__global__ void gate_heads_kernel(act_t* __restrict__ o, const act_t* __restrict__ g, int ldg, int W, int per) {
   const int t = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= W) return;
-  const float z = to_f32(g[(size_t)t * ldg + i]);
+  const float z = to_f32(g[(size_t)t * ldg + i / per]);
   const size_t at = (size_t)t * W + i;
   o[at] = from_f32<act_t>(to_f32(o[at]) / (1.0f + expf(-z)));
 }
@@ -39,16 +40,22 @@ int zk_unary_act(const void* x, void* out, size_t n, int act, void* stream) {
 }
 
 // o: [T, W] activations, multiplied in place by sigmoid(g[t, i]); g: rows ldg apart.
-int zk_gate_heads(void* o, const void* g, int ldg, int T, int W, void* stream) {
-  ZK_REQUIRE(T >= 0 && W > 0 && ldg >= W && g != nullptr, "zk_gate_heads: bad sizes");
+// per: the channels that share one gate value (1: a value a channel; a head's size: a value a head).
+int zk_gate_heads_per(void* o, const void* g, int ldg, int T, int W, int per, void* stream) {
+  ZK_REQUIRE(T >= 0 && W > 0 && per > 0 && W % per == 0 && ldg >= W / per && g != nullptr, "zk_gate_heads: bad sizes");
   ZK_REQUIRE(T <= 65535, "zk_gate_heads: more than 65535 rows");
   if (T == 0) return 0;
   dim3 grid((W + 255) / 256, T);
-  gate_heads_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((act_t*)o, (const act_t*)g, ldg, W);
+  gate_heads_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((act_t*)o, (const act_t*)g, ldg, W, per);
   return zk_launch_status("zk_gate_heads");
+}
+
+int zk_gate_heads(void* o, const void* g, int ldg, int T, int W, void* stream) {
+  return zk_gate_heads_per(o, g, ldg, T, W, 1, stream);
 }
 
 }  // extern "C"
 
 ZK_ENTER(zk_unary_act)
 ZK_ENTER(zk_gate_heads)
+ZK_ENTER(zk_gate_heads_per)

@@ -44,6 +44,40 @@ __global__ void sum_norm_kernel(float* __restrict__ h, const void* __restrict__ 
     out[row + i] = from_f32<act_t>(hr[i] * inv * (unit_offset ? 1.0f + w_next[i] : w_next[i]));
 }
 
+// h <- h + (a + b + bias); out = layer_norm(h) = (h - mean) / sqrt(var + eps) * w + c, var the mean of
+// the squared deviations (two passes over the row: the mean first, then the deviations)
+__global__ void sum_layer_norm_kernel(float* __restrict__ h, const void* __restrict__ a, int a_parts,
+                                      const void* __restrict__ b, int b_parts, const float* __restrict__ bias,
+                                      const float* __restrict__ w_next, const float* __restrict__ c_next, float eps,
+                                      act_t* __restrict__ out, int W) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const size_t plane = (size_t)gridDim.x * W, row = (size_t)r * W;
+  float* hr = h + row;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v = hr[i];
+    if (a != nullptr || b != nullptr || bias != nullptr) {
+      float y = planes_value(a, a_parts, plane, row + i) + planes_value(b, b_parts, plane, row + i);
+      if (bias) y += bias[i];
+      v += y;
+      hr[i] = v;
+    }
+    s += v;
+  }
+  if (!w_next) return;
+  const float mean = block_sum(s, red) / (float)W;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {      // each thread re-reads what it wrote
+    const float d = hr[i] - mean;
+    ss = fmaf(d, d, ss);
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x)
+    out[row + i] = from_f32<act_t>((hr[i] - mean) * inv * w_next[i] + (c_next ? c_next[i] : 0.f));
+}
+
 // h <- h + mult * (a + b + bias); out1 = norm(h) * gain1, out2 = norm(h) * gain2: a layer whose two
 // sublayers read two norms of the same stream (either output may be absent)
 __global__ void sum_norm_pair_kernel(float* __restrict__ h, const void* __restrict__ a, int a_parts,
@@ -116,6 +150,18 @@ int zk_sum_norm(float* h, const void* a, int a_parts, const void* b, int b_parts
   return zk_launch_status("zk_sum_norm");
 }
 
+// As zk_sum_norm with a layer norm of the new stream: gain w_next, bias c_next (may be null).
+// a, b and bias all null: the stream stays as it is and only the norm is made.
+int zk_sum_layer_norm(float* h, const void* a, int a_parts, const void* b, int b_parts, const float* bias,
+                      const float* w_next, const float* c_next, float eps, void* out, int T, int W, void* stream) {
+  ZK_REQUIRE(T >= 0 && W > 0 && a_parts >= 0 && b_parts >= 0, "zk_sum_layer_norm: bad sizes");
+  ZK_REQUIRE(w_next == nullptr || out != nullptr, "zk_sum_layer_norm: a norm without output");
+  if (T == 0) return 0;
+  sum_layer_norm_kernel<<<T, 256, 0, (hipStream_t)stream>>>(h, a, a_parts, b, b_parts, bias, w_next, c_next, eps,
+                                                           (act_t*)out, W);
+  return zk_launch_status("zk_sum_layer_norm");
+}
+
 // As zk_sum_norm, with the sublayers' sum times ``mult`` and up to two norms of the new stream
 // (w1 -> out1, w2 -> out2; either pair may be null).  a, b and bias all null: the stream stays as
 // it is and only the norms are made.
@@ -159,6 +205,7 @@ int zk_planes_sum(const float* planes, int parts, void* out, int T, int W, void*
 }  // extern "C"
 
 ZK_ENTER(zk_sum_norm)
+ZK_ENTER(zk_sum_layer_norm)
 ZK_ENTER(zk_sum_norm_pair)
 ZK_ENTER(zk_weighted_sum)
 ZK_ENTER(zk_add_bias)

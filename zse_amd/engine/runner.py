@@ -217,6 +217,12 @@ class StepRunner:
                 cc.extra[key] = (slot_bytes, int(nbytes))
                 slot_bytes += (int(nbytes) + 15) // 16 * 16
             self.caches.append(cc)
+        # what the embedding keeps per request (the last token, for a table of token pairs)
+        self.embedding_state = None
+        emb_bytes = int(model.embedding.state_bytes()) if hasattr(model.embedding, "state_bytes") else 0
+        if emb_bytes:
+            self.embedding_state = (slot_bytes, emb_bytes)
+            slot_bytes += (emb_bytes + 15) // 16 * 16
         self.slot_bytes = slot_bytes
         self.manager = CacheManager(groups, self.page_size, self.max_seqs, self.max_model_len, slot_bytes,
                                     first_page=1)
@@ -435,6 +441,7 @@ class StepRunner:
         ctx.entries = host_entries
         ctx.max_q_len, ctx.max_ctx, ctx.n_multi = max_q, max_ctx, n_multi
         ctx.state, ctx.slot_bytes = self.state, self.slot_bytes
+        ctx.embedding_state = self.embedding_state
         return ctx
 
     def _ensure_logits(self, rows: int):

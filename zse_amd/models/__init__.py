@@ -1,2 +1,2 @@
 """Importing this package registers every architecture the engine serves."""
-from . import bumolix, dafotar, gemma2, pubunex  # noqa: F401
+from . import bumolix, dafotar, gemma2, pubunex, rotalorn  # noqa: F401

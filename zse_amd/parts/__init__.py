@@ -1,5 +1,5 @@
 """Parts a model is put together from.  Importing the package registers the built-in kinds."""
-from . import (attention, block, delta, embedding, ffn, gla, latent, mlstm, norm, position, scan, shortconv,  # noqa: F401
+from . import (attention, block, delta, diffattn, embedding, ffn, gla, latent, mlstm, norm, position, scan, shortconv,  # noqa: F401
                sidebyside, streams)
 from .base import (PagedKV, Part, StateNeed, TensorReq, build_part, register_part,
                    unregister_part, walk)

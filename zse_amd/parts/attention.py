@@ -48,6 +48,11 @@ class PagedAttention(Part):
         self.unit_norm = bool(getattr(s, "qk_unit_norm", False))
         self.gate_name = getattr(s, "gate", None)
         self.wide_weights = bool(getattr(s, "wide_weights", False))
+        # a norm over a token's whole query row and whole key row, and values that are the keys as
+        # projected: one kernel of their own between the product and the attention
+        self.q_row_norm_name, self.k_row_norm_name = getattr(s, "q_row_norm", None), getattr(s, "k_row_norm", None)
+        self.values_are_keys = bool(getattr(s, "values_are_keys", False))
+        self.by_rows = bool(self.q_row_norm_name or self.k_row_norm_name or self.values_are_keys)
         if self.chunk and s.window:
             raise ValueError("an attention has a window or a chunk, not both")
         if self.chunk < 0:
@@ -55,13 +60,23 @@ class PagedAttention(Part):
         self.general = bool(self.value_dim != s.head_dim or self.q_norm_name or self.k_norm_name or
                             self.head_scale_name or self.value_base or self.bias_names or
                             self.rot_scale != 1.0 or self.rot_interleaved or self.chunk or self.unit_sink or self.wide_weights or
-                            self.unit_norm or self.gate_name)
+                            self.unit_norm or self.gate_name or self.by_rows)
+        if self.by_rows:
+            if (self.q_norm_name or self.k_norm_name or self.head_scale_name or self.value_base or self.unit_norm
+                    or self.rot_scale != 1.0 or self.rot_interleaved or self.shared_kv):
+                raise ValueError("an attention with norms over whole rows, or whose values are its keys, takes biases, "
+                                 "a rotation of pairs (i, i + dims/2), a window or chunk, a sink and a gate, nothing else")
+            if self.values_are_keys and self.value_dim != s.head_dim:
+                raise ValueError(f"values that are keys have the keys' size: value_dim {self.value_dim}, head_dim {s.head_dim}")
+            if self.values_are_keys and ("v" in s.names or "v" in self.bias_names):
+                raise ValueError("values that are keys have no projection and no bias of their own")
         self.in_bias = self.o_bias = None
         if self.value_dim > 256:
             raise ValueError(f"value_dim up to 256, got {self.value_dim}")
         if self.value_base and self.value_dim % 2:
             raise ValueError(f"rotated values need an even value_dim, got {self.value_dim}")
         self.q_gain = self.k_gain = self.head_scale = self.value_freq = None
+        self.q_row_gain = self.k_row_gain = None
         self.decode_chunk = 64                     # keys a wave of the split decode attention takes
 
     def children(self):
@@ -80,20 +95,26 @@ class PagedAttention(Part):
         for role, rows in (("q", s.num_heads * s.head_dim), ("o", s.hidden_size)):
             if role in self.bias_names:
                 out.append(TensorReq(self.bias_names[role], (rows,), ROLE_GAIN))
+        if self.q_row_norm_name:
+            out.append(TensorReq(self.q_row_norm_name, (s.num_heads * s.head_dim,), ROLE_GAIN))
         if self.shared_kv:
             return out
         for role, rows in (("k", s.num_kv_heads * s.head_dim), ("v", s.num_kv_heads * self.value_dim)):
             if role in self.bias_names:
                 out.append(TensorReq(self.bias_names[role], (rows,), ROLE_GAIN))
-        out += [TensorReq(s.names["k"], (s.num_kv_heads * s.head_dim, s.hidden_size)),
-                TensorReq(s.names["v"], (s.num_kv_heads * self.value_dim, s.hidden_size))]
+        out.append(TensorReq(s.names["k"], (s.num_kv_heads * s.head_dim, s.hidden_size)))
+        if not self.values_are_keys:
+            out.append(TensorReq(s.names["v"], (s.num_kv_heads * self.value_dim, s.hidden_size)))
+        if self.k_row_norm_name:
+            out.append(TensorReq(self.k_row_norm_name, (s.num_kv_heads * s.head_dim,), ROLE_GAIN))
         if self.k_norm_name:
             out.append(TensorReq(self.k_norm_name, (s.head_dim,), ROLE_GAIN))
         return out
 
     def load(self, weights, rt, dtype):
         s = self.spec
-        names = [s.names["q"]] if self.shared_kv else [s.names[r] for r in ("q", "k", "v")]
+        stored = ("q", "k") if self.values_are_keys else ("q", "k", "v")
+        names = [s.names["q"]] if self.shared_kv else [s.names[r] for r in stored]
         if self.gate_name:
             names.append(self.gate_name)       # the gate's rows behind q, k, v: one product
         strip = getattr(weights, "wants_strip", None)
@@ -107,7 +128,11 @@ class PagedAttention(Part):
             self.k_gain = weights.vector(self.k_norm_name)
         if self.head_scale_name:
             self.head_scale = weights.vector(self.head_scale_name)
-        roles = ("q",) if self.shared_kv else ("q", "k", "v")
+        if self.q_row_norm_name:
+            self.q_row_gain = weights.vector(self.q_row_norm_name)
+        if self.k_row_norm_name:
+            self.k_row_gain = weights.vector(self.k_row_norm_name)
+        roles = ("q",) if self.shared_kv else stored
         if any(r in self.bias_names for r in roles):
             if not all(r in self.bias_names for r in roles):
                 raise ValueError("biases on the projections: all of q, k, v or none")
@@ -178,7 +203,7 @@ class PagedAttention(Part):
         T = x.shape[0]
         nh, nkv, hd, vd = s.num_heads, s.num_kv_heads, s.head_dim, self.value_dim
         n_store = 0 if self.shared_kv else nkv
-        heads_width = (nh + n_store) * hd + n_store * vd
+        heads_width = (nh + n_store) * hd + (0 if self.values_are_keys else n_store * vd)
         width = heads_width + (nh * vd if self.gate_name else 0)
         g = ctx.group(cache.group)
         tables = self.position.rotary_tables()
@@ -188,13 +213,21 @@ class PagedAttention(Part):
         ptr = lambda t: t.ptr if t is not None else None
         vfreq = ptr(self.value_freq)
         inter = 1 if getattr(s, "value_pairs_interleaved", False) else 0
-        prep = (qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map, ptr(self.q_gain),
+        if self.by_rows:
+            # bias, the norms over whole rows, rotation and the store of keys and values, one launch
+            k.zk_row_prep(qkv.ptr, width, ctx.positions, g.slot_map, ptr(self.in_bias), ptr(self.q_row_gain),
+                          ptr(self.k_row_gain), float(s.norm_eps), tables[0].ptr if tables is not None else None,
+                          tables[1] if tables is not None else 0, cache.k.ptr, cache.v.ptr, T, nh, nkv, hd, vd,
+                          g.page_size, 1 if cache.v_transposed else 0, 1 if self.values_are_keys else 0, ctx.stream)
+        prep = None if self.by_rows else (qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map, ptr(self.q_gain),
                 ptr(self.k_gain), ptr(self.head_scale), float(s.norm_eps),
                 tables[0].ptr if tables is not None else None, tables[1] if tables is not None else 0, vfreq,
                 inter, cache.k.ptr, cache.v.ptr, T, nh, n_store, hd, vd, g.page_size,
                 1 if cache.v_transposed else 0, ptr(self.in_bias), self.rot_scale,
                 1 if self.rot_interleaved else 0)
-        if self.unit_norm or width != heads_width:
+        if prep is None:
+            pass
+        elif self.unit_norm or width != heads_width:
             k.zk_head_prep_unit(*prep, width, 1 if self.unit_norm else 0, ctx.stream)
         else:
             k.zk_head_prep_ext(*prep, ctx.stream)

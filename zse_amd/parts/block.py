@@ -10,7 +10,7 @@ from __future__ import annotations
 
 from ..runtime.device import Tensor
 from .base import Part, build_part, register_part
-from .norm import RMSNorm
+from .norm import LayerNorm, RMSNorm
 
 ARRANGEMENTS = {"sandwich": ("pre_mixer", "post_mixer", "pre_ffn", "post_ffn"),
                 "prenorm": ("pre_mixer", "pre_ffn")}
@@ -91,7 +91,8 @@ class ParallelBlock(Part):
     are summed before they join it (``ffn`` None: the mixer alone).  With a second norm
     ``pre_ffn`` the feed-forward reads that norm of the same h instead, and with
     ``residual_scale`` m the sum joins as h += m (mixer + ffn).  One kernel does the sum, the
-    mixer's output bias if it has one, the residual sum and the norms of whatever runs next."""
+    mixer's output bias if it has one, the residual sum and the norms of whatever runs next (RMS
+    norms, or one layer norm with gain and bias over a single stream)."""
     graph_safe = True      # its launches take what changes from step to step from device memory alone
 
     def __init__(self, spec):
@@ -153,7 +154,8 @@ class ParallelBlock(Part):
             m = self.ffn.forward(ctx, x2 if x2 is not None else x)
             ctx.sums_welcome = None
         nxt = next_norm if isinstance(next_norm, tuple) else ((next_norm,) if next_norm is not None else ())
-        if not nxt or not self._fusable(nxt) or len(nxt) > 2:
+        layer_norm = (len(nxt) == 1 and isinstance(nxt[0], LayerNorm) and nxt[0].spec.streams == 1 and self.mult == 1.0)
+        if not nxt or not (self._fusable(nxt) or layer_norm) or len(nxt) > 2:
             nxt = ()             # norms the closing kernel does not know: the next block applies them
         outs = []
         for i in range(len(nxt)):
@@ -161,7 +163,11 @@ class ParallelBlock(Part):
             outs.append(ctx.alloc((T, H)) if buf is None else Tensor(buf.ptr, (T, H), ctx.dtype, buf.owner))
         planes = lambda t: t.shape[0] if (t is not None and t.layout == "parts") else 0
         ptr = lambda t: t.ptr if t is not None else None
-        if self.mult == 1.0 and len(nxt) <= 1:
+        if nxt and layer_norm:
+            n0 = nxt[0]
+            ctx.k.zk_sum_layer_norm(h.ptr, a.ptr, planes(a), ptr(m), planes(m), ptr(bias), n0.weight.ptr, ptr(n0.bias),
+                                    float(n0.spec.eps), outs[0].ptr, T, H, ctx.stream)
+        elif self.mult == 1.0 and len(nxt) <= 1:
             ns = nxt[0].spec if nxt else None
             ctx.k.zk_sum_norm(h.ptr, a.ptr, planes(a), ptr(m), planes(m), ptr(bias), nxt[0].weight.ptr if nxt else None,
                               float(ns.eps) if ns is not None else 0.0, int(ns.unit_offset) if ns is not None else 0,

@@ -27,9 +27,22 @@ class Embedding(Part):
         self.scale = float(spec.scale)
 
     def tensor_reqs(self) -> List[TensorReq]:
-        return [TensorReq(self.spec.weight, (self.spec.vocab_size, self.spec.hidden_size))]
+        out = [TensorReq(self.spec.weight, (self.spec.vocab_size, self.spec.hidden_size))]
+        pairs = getattr(self.spec, "pairs", None)
+        if pairs is not None:
+            out.append(TensorReq(pairs.weight, (pairs.buckets + 1, self.spec.hidden_size)))
+        return out
+
+    def state_bytes(self) -> int:
+        """What the embedding keeps per request: with a table of token pairs, the request's last token."""
+        return 4 if getattr(self.spec, "pairs", None) is not None else 0
 
     def load(self, weights, rt, dtype):
+        pairs = getattr(self.spec, "pairs", None)
+        if pairs is not None:
+            if pairs.buckets < 1:
+                raise ValueError(f"a pair table needs at least one bucket, got {pairs.buckets}")
+            self.pair_table = weights.matrix([pairs.weight])          # row-major: rows are gathered
         # the table may be the head's matrix too (tied): both ask for the same layout
         strip = getattr(weights, "wants_strip", None)
         self.table = (weights.matrix([self.spec.weight], strip=True) if strip and strip(self.spec.hidden_size)
@@ -52,6 +65,19 @@ class Embedding(Part):
         row = h if copies == 1 else ctx.alloc((ctx.T, s.hidden_size), F32)
         ctx.k.zk_embed(self.table.ptr, ctx.tokens, row.ptr, self.scale, ctx.T, s.hidden_size,
                        s.vocab_size, 1 if self.table.layout == "strip" else 0, ctx.stream)
+        pairs = getattr(s, "pairs", None)
+        if pairs is not None:
+            # the token before each request's first of this step comes from its state slot, where
+            # the request's last token of this step takes its place
+            place = getattr(ctx, "embedding_state", None)
+            if place is None or ctx.state is None:
+                raise RuntimeError("an embedding with a pair table needs a place in the requests' state slots")
+            before = ctx.alloc((max(ctx.R, 1),), "int32")
+            ctx.k.zk_prev_token(ctx.tokens, ctx.q_start, ctx.slot_of_req, ctx.state.ptr, ctx.slot_bytes // 4,
+                                place[0] // 4, before.ptr, ctx.R, ctx.stream)
+            ctx.k.zk_add_pair_rows(row.ptr, self.pair_table.ptr, ctx.tokens, ctx.positions, ctx.req_of_token, ctx.q_start,
+                                   before.ptr, pairs.buckets, pairs.mul_prev, pairs.mul_cur, ctx.T, s.hidden_size,
+                                   ctx.stream)
         if copies > 1:          # every residual stream starts as the embedded row
             ctx.k.zk_replicate(row.ptr, h.ptr, ctx.T, copies, s.hidden_size, ctx.stream)
         return h

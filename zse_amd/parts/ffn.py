@@ -59,15 +59,13 @@ class GatedMLP(Part):
             a = ctx.alloc((T, I))
             ctx.k.zk_clamped_glu(gu.ptr, a.ptr, T, I, float(s.limit), ctx.stream)
             return linear(ctx, a, self.w_down, out if out is not None else ctx.alloc((T, s.hidden_size)), last_of=last)
-        if out is not None:
-            raise ValueError("a result buffer of the caller's is taken by the clamped layer only")
         if tuned_gemm(ctx, s.hidden_size):
             a = linear(ctx, x, self.w_gu, ctx.alloc((T, I)), epilogue=s.activation)
-            return linear(ctx, a, self.w_down, ctx.alloc((T, s.hidden_size)), last_of=self)
+            return linear(ctx, a, self.w_down, out if out is not None else ctx.alloc((T, s.hidden_size)), last_of=last)
         gu = linear(ctx, x, self.w_gu, ctx.alloc((T, 2 * I)))
         a = ctx.alloc((T, I))
         ctx.k.zk_gated_act(gu.ptr, a.ptr, T, I, ACTIVATION_CODES[s.activation], ctx.stream)
-        return linear(ctx, a, self.w_down, ctx.alloc((T, s.hidden_size)), last_of=self)
+        return linear(ctx, a, self.w_down, out if out is not None else ctx.alloc((T, s.hidden_size)), last_of=last)
 
 
 UNARY_CODES = {"relu2": 0}     # max(z, 0)^2
@@ -108,10 +106,11 @@ class MLP(Part):
 
 
 class RoutedMLP(Part):
-    """A mixture of small gated layers: sigmoid scores from a float router product, the ``top_k``
-    largest chosen on the device (the lower index among equals), the chosen scores as weights on
-    the experts' inputs, the experts' results added in the order they were chosen, a shared layer
-    on top.  Steps of few tokens read each chosen expert's rows once per (token, choice); steps of
+    """A mixture of small gated layers: scores from a float router product (sigmoids, or a softmax
+    over all experts), the ``top_k`` largest chosen on the device (the lower index among equals),
+    the chosen scores as weights on the experts' inputs or on their outputs, the experts' results
+    added in the order they were chosen, a shared layer on top (optionally times the sigmoid of a
+    number a token, whose row rides below the router's in one product).  Steps of few tokens read each chosen expert's rows once per (token, choice); steps of
     many tokens sort the pairs by expert on the device and run a grouped matrix-core product.
     Nothing comes back to the host, so steps are captured and written down like any other."""
     graph_safe = True
@@ -123,15 +122,19 @@ class RoutedMLP(Part):
 
     def __init__(self, spec):
         s = self.spec = spec
-        if s.activation != CLAMPED:
-            raise ValueError(f"routed experts are {CLAMPED} layers, got {s.activation!r}")
+        if s.activation not in (CLAMPED, "silu"):
+            raise ValueError(f"routed experts are {CLAMPED} or silu layers, got {s.activation!r}")
         if not (1 <= s.top_k <= min(s.num_experts, 16)) or s.num_experts > 1024:
             raise ValueError(f"1 to 16 of up to 1024 experts a token, got {s.top_k} of {s.num_experts}")
-        if not s.scale_input:
-            raise ValueError("routed experts take their weight on the input")
-        if not (s.limit or 0) > 0:
+        if s.activation == CLAMPED and not (s.limit or 0) > 0:
             raise ValueError(f"{CLAMPED} needs a positive limit, got {s.limit!r}")
+        self.scoring = getattr(s, "scoring", "sigmoid")
+        if self.scoring not in ("sigmoid", "softmax"):
+            raise ValueError(f"scores are sigmoid or softmax, got {self.scoring!r}")
         self.shared = build_part("ffn", s.shared) if s.shared is not None else None
+        self.shared_gate = getattr(s, "shared_gate", None)
+        if self.shared_gate and self.shared is None:
+            raise ValueError("a gate on the shared layer needs a shared layer")
         self.w_router = self.w_gu = self.w_down = None
 
     def children(self):
@@ -143,6 +146,8 @@ class RoutedMLP(Part):
     def tensor_reqs(self) -> List[TensorReq]:
         s = self.spec
         out = [TensorReq(s.router, (s.num_experts, s.hidden_size))]
+        if self.shared_gate:
+            out.append(TensorReq(self.shared_gate, (1, s.hidden_size)))
         for e in range(s.num_experts):
             out += [TensorReq(self._name(e, "gate"), (s.intermediate_size, s.hidden_size)),
                     TensorReq(self._name(e, "up"), (s.intermediate_size, s.hidden_size)),
@@ -151,7 +156,7 @@ class RoutedMLP(Part):
 
     def load(self, weights, rt, dtype):
         s = self.spec
-        self.w_router = weights.matrix([s.router])
+        self.w_router = weights.matrix([s.router] + ([self.shared_gate] if self.shared_gate else []))
         # expert e: rows [e 2F, e 2F + F) its gate, the next F its up; down: rows [e W, (e + 1) W)
         self.w_gu = weights.matrix([self._name(e, r) for e in range(s.num_experts) for r in ("gate", "up")])
         self.w_down = weights.matrix([self._name(e, "down") for e in range(s.num_experts)])
@@ -163,25 +168,30 @@ class RoutedMLP(Part):
     def forward(self, ctx, x: Tensor) -> Tensor:
         s, k = self.spec, ctx.k
         T, W, F, E, top = x.shape[0], s.hidden_size, s.intermediate_size, s.num_experts, s.top_k
-        logits = linear(ctx, x, self.w_router, ctx.alloc((T, E), F32))
+        ld = E + (1 if self.shared_gate else 0)
+        logits = linear(ctx, x, self.w_router, ctx.alloc((T, ld), F32))
         ids, wts = ctx.alloc((T, top), I32), ctx.alloc((T, top), F32)
-        k.zk_moe_route(logits.ptr, ids.ptr, wts.ptr, T, E, top, ctx.stream)
+        k.zk_moe_route_ext(logits.ptr, ld, ids.ptr, wts.ptr, T, E, top, 1 if self.scoring == "softmax" else 0, ctx.stream)
+        act, on_out, limit = (1 if s.activation == "silu" else 0), (0 if s.scale_input else 1), float(s.limit or 0.0)
         P = 2 if self.shared is not None else 1
         planes = ctx.alloc((P, T, W), F32)
         y = ctx.alloc((T * top, F))
         enough = T * top >= (self.GROUPED_WIDE_FROM if W * F >= self.WIDE else self.GROUPED_FROM)
         grouped = (ctx.dtype == BF16 and ctx.tuned and enough and W % 8 == 0 and F % 8 == 0
-                   and k.has("zk_moe_experts_grouped"))
+                   and k.has("zk_moe_experts_grouped_ext"))
         if grouped:
             work = ctx.alloc((E + 1 + 2 * T * top,), I32)
             xg, rows = ctx.alloc((T * top, W)), ctx.alloc((T * top, W), F32)
-            k.zk_moe_experts_grouped(x.ptr, ids.ptr, wts.ptr, self.w_gu.ptr, self.w_down.ptr, work.ptr, xg.ptr, y.ptr,
-                                     rows.ptr, planes.ptr, T, E, top, W, F, float(s.limit), ctx.stream)
+            k.zk_moe_experts_grouped_ext(x.ptr, ids.ptr, wts.ptr, self.w_gu.ptr, self.w_down.ptr, work.ptr, xg.ptr, y.ptr,
+                                         rows.ptr, planes.ptr, T, E, top, W, F, limit, act, on_out, ctx.stream)
         else:
-            k.zk_moe_experts(x.ptr, ids.ptr, wts.ptr, self.w_gu.ptr, self.w_down.ptr, y.ptr, planes.ptr, T, top, W, F,
-                             float(s.limit), ctx.stream)
+            k.zk_moe_experts_ext(x.ptr, ids.ptr, wts.ptr, self.w_gu.ptr, self.w_down.ptr, y.ptr, planes.ptr, T, top, W, F,
+                                 limit, act, on_out, ctx.stream)
         if self.shared is not None:
-            self.shared.forward(ctx, x, out=planes.rows(1, 2).view(T, W))
+            second = planes.rows(1, 2).view(T, W)
+            self.shared.forward(ctx, x, out=second)
+            if self.shared_gate:
+                k.zk_gate_rows(second.ptr, logits.ptr + E * 4, ld, T, W, ctx.stream)
         if getattr(ctx, "sums_welcome", None) is self:
             # the block's joining kernel adds the planes up itself
             return Tensor(planes.ptr, (P, T, W), F32, planes.owner, layout="parts")

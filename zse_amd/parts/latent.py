@@ -10,12 +10,16 @@ head is carried over to [W_uk,h^T q_plain, q_rot], attends to the cached rows as
 first C channels as values, and its result goes through W_uv,h; the two small per-head products
 run before and after the attention kernel.  One path for whole prompts, portions and decoded
 tokens, reading the cache alone.
+
+Options of the spec: queries through a latent of their own (c_q = rms_norm(W_q_down x) * gain,
+q = W_q c_q), a window over the keys, and a gate of one number a head, sigmoid(W_gate x)_h, on the
+heads' outputs (its rows ride behind the down-projection's in one product).
 """
 from __future__ import annotations
 
 from typing import List
 
-from ..runtime.device import BF16, Tensor
+from ..runtime.device import BF16, ITEMSIZE, Tensor
 from .base import ROLE_GAIN, PagedKV, Part, TensorReq, build_part, register_part
 from .ops import linear
 
@@ -34,6 +38,11 @@ class LatentAttention(Part):
             raise ValueError("a latent attention's rotated part needs a rotary encoding over all of its channels")
         self.w_in = self.w_uk = self.w_uv = self.w_o = None
         self.gain = self.sinks = None
+        self.q_rank = int(getattr(s, "query_latent_dim", None) or 0)
+        self.gate_name = s.names.get("gate")
+        if self.q_rank and not (s.names.get("q_down") and s.names.get("q_down_norm")):
+            raise ValueError("queries through a latent need the tensors q_down and q_down_norm")
+        self.w_q_down = self.w_q = self.q_gain = None
 
     def children(self):
         return [self.position]
@@ -41,17 +50,30 @@ class LatentAttention(Part):
     def tensor_reqs(self) -> List[TensorReq]:
         s, n = self.spec, self.spec.names
         H, D, R, E, C, W = s.num_heads, s.head_dim, s.rotary_dim, s.value_dim, s.latent_dim, s.hidden_size
-        out = [TensorReq(n["q"], (H * (D + R), W)), TensorReq(n["down"], (C + R, W)),
+        out = [TensorReq(n["q"], (H * (D + R), self.q_rank or W)), TensorReq(n["down"], (C + R, W)),
                TensorReq(n["down_norm"], (C,), ROLE_GAIN), TensorReq(n["up_k"], (H * D, C)),
                TensorReq(n["up_v"], (H * E, C)), TensorReq(n["o"], (W, H * E))]
         if n.get("sinks"):
             out.append(TensorReq(n["sinks"], (H,), ROLE_GAIN))
+        if self.q_rank:
+            out += [TensorReq(n["q_down"], (self.q_rank, W)), TensorReq(n["q_down_norm"], (self.q_rank,), ROLE_GAIN)]
+        if self.gate_name:
+            out.append(TensorReq(self.gate_name, (H, W)))
         return out
 
     def load(self, weights, rt, dtype):
         s, n = self.spec, self.spec.names
         strip = getattr(weights, "wants_strip", None)
-        self.w_in = weights.matrix([n["q"], n["down"]], strip=bool(strip and strip(s.hidden_size)))
+        tail = [n["down"]] + ([self.gate_name] if self.gate_name else [])
+        if self.q_rank:
+            # the query's own latent is a product, a norm and a second product; the down-projection
+            # (and the gate) is a product of its own
+            self.w_q_down = weights.matrix([n["q_down"]], strip=bool(strip and strip(s.hidden_size)))
+            self.w_q = weights.matrix([n["q"]], strip=bool(strip and strip(self.q_rank)))
+            self.q_gain = weights.vector(n["q_down_norm"])
+            self.w_in = weights.matrix(tail, strip=bool(strip and strip(s.hidden_size)))
+        else:
+            self.w_in = weights.matrix([n["q"]] + tail, strip=bool(strip and strip(s.hidden_size)))
         self.w_uk, self.w_uv = weights.matrix([n["up_k"]]), weights.matrix([n["up_v"]])      # row-major: read per head
         self.w_o = weights.matrix([n["o"]], strip=bool(strip and strip(s.num_heads * s.value_dim)))
         self.gain = weights.vector(n["down_norm"])
@@ -88,15 +110,28 @@ class LatentAttention(Part):
         s, k = self.spec, ctx.k
         T = x.shape[0]
         H, D, R, E, C = s.num_heads, s.head_dim, s.rotary_dim, s.value_dim, s.latent_dim
-        ld = H * (D + R) + C + R
         g = ctx.group(cache.group)
-        qd = linear(ctx, x, self.w_in, ctx.alloc((T, ld)))
+        item = ITEMSIZE[ctx.dtype]
+        n_gate = H if self.gate_name else 0
+        if self.q_rank:
+            cq = linear(ctx, x, self.w_q_down, ctx.alloc((T, self.q_rank)))
+            cn = ctx.alloc((T, self.q_rank))
+            k.zk_rmsnorm(cq.ptr, 0, None, self.q_gain.ptr, cn.ptr, float(s.eps), 0, T, self.q_rank, ctx.stream)
+            qd = linear(ctx, cn, self.w_q, ctx.alloc((T, H * (D + R))))
+            ld = H * (D + R)
+            ldd = C + R + n_gate
+            down = linear(ctx, x, self.w_in, ctx.alloc((T, ldd)))
+            down_ptr = down.ptr
+        else:
+            ld = ldd = H * (D + R) + C + R + n_gate
+            qd = linear(ctx, x, self.w_in, ctx.alloc((T, ld)))
+            down_ptr = qd.ptr + H * (D + R) * item
         qa = ctx.alloc((T, H * (C + R)))
         tables = self.position.rotary_tables()
         mag = float(self.position.magnitude()) if hasattr(self.position, "magnitude") else 1.0
         inter = 1 if getattr(self.position, "interleaved", False) else 0
-        k.zk_latent_prep(qd.ptr, ld, ctx.positions, g.slot_map, self.gain.ptr, float(s.eps), tables[0].ptr, mag, inter,
-                         qa.ptr, cache.k.ptr, T, H, D, R, C, g.page_size, ctx.stream)
+        k.zk_latent_prep_ext(qd.ptr, ld, down_ptr, ldd, ctx.positions, g.slot_map, self.gain.ptr, float(s.eps),
+                             tables[0].ptr, mag, inter, qa.ptr, cache.k.ptr, T, H, D, R, C, g.page_size, ctx.stream)
         # the plain part of every query head, carried over to the latent's channels
         k.zk_heads_linear(qd.ptr, ld, D + R, self.w_uk.ptr, 1, qa.ptr, H * (C + R), C + R, T, H, D, C, ctx.stream)
         o = ctx.alloc((T, H * C))
@@ -112,6 +147,9 @@ class LatentAttention(Part):
                                       float(s.scale), 0.0, int(s.window) if s.window else 0, 0, None, 0, sinks, 1, ctx.stream)
         v = ctx.alloc((T, H * E))
         k.zk_heads_linear(o.ptr, H * C, C, self.w_uv.ptr, 0, v.ptr, H * E, E, T, H, C, E, ctx.stream)
+        if self.gate_name:
+            # a head's output times the sigmoid of its gate column, which lies behind the down-projection's
+            k.zk_gate_heads_per(v.ptr, down_ptr + (C + R) * item, ldd, T, H * E, E, ctx.stream)
         return linear(ctx, v, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)
 
 

@@ -23,6 +23,9 @@ class Rotary(Part):
             raise ValueError(f"rotary_dim must be even and in (0, head_dim], got {spec.rotary_dim}")
         if getattr(spec, "linear_factor", None) is not None and not spec.linear_factor > 0:
             raise ValueError(f"linear_factor must be positive, got {spec.linear_factor}")
+        ws = getattr(spec, "wavelength_scaling", None)
+        if ws is not None and not (ws[0] > 0 and ws[3] > 0 and ws[1] > 0 and ws[2] > ws[1]):
+            raise ValueError(f"wavelength_scaling needs factor, original > 0 and high > low > 0, got {ws}")
         self.spec = spec
         self.inv_freq = None
 
@@ -43,6 +46,17 @@ class Rotary(Part):
         linear = getattr(s, "linear_factor", None)
         if linear is not None:
             f = f / float(linear)
+        by_wavelength = getattr(s, "wavelength_scaling", None)
+        if by_wavelength is not None:
+            # each frequency on its own, by how its wavelength compares with the original length
+            factor, low, high, original = (float(v) for v in by_wavelength)
+            for n in range(len(f)):
+                length = 2.0 * math.pi / f[n]
+                if length > original / low:
+                    f[n] = f[n] / factor
+                elif length >= original / high:
+                    share = (original / length - low) / (high - low)
+                    f[n] = (1.0 - share) * f[n] / factor + share * f[n]
         return f.astype(np.float32)
 
     def magnitude(self) -> float:

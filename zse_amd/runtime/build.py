@@ -28,7 +28,7 @@ ARCH = "gfx950"
 
 COMMON_KERNELS = ["elementwise.hip", "gemm_plain.hip", "attention_plain.hip", "sampling.hip", "probe.hip", "steplist.hip",
                   "streams.hip", "headprep.hip", "mlstm.hip", "delta.hip", "moe.hip", "latent.hip", "residual.hip", "gla.hip", "scan.hip",
-                  "pointwise.hip"]
+                  "pointwise.hip", "embed_pair.hip", "diffattn.hip"]
 BF16_KERNELS = ["gemm_bf16.hip", "attention_bf16.hip"]
 
 LIBRARIES: Dict[str, dict] = {

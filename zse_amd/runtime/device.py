@@ -205,6 +205,19 @@ KERNEL_SIGNATURES = {
     "zk_gate_heads": [_VP, _VP, _I, _I, _I, _VP],
     "zk_gla": [_VP, _I, _I, _I, _VP, _I, _VP, _I, _VP, _F, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I,
                _F, _I, _VP, _VP, _VP],
+    "zk_prev_token": [_VP, _VP, _VP, _VP, _SZ, _SZ, _VP, _I, _VP],
+    "zk_add_pair_rows": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "zk_row_prep": [_VP, _I, _VP, _VP, _VP, _VP, _VP, _F, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_latent_prep_ext": [_VP, _I, _VP, _I, _VP, _VP, _VP, _F, _VP, _F, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_gate_heads_per": [_VP, _VP, _I, _I, _I, _I, _VP],
+    "zk_sum_layer_norm": [_VP, _VP, _I, _VP, _I, _VP, _VP, _VP, _F, _VP, _I, _I, _VP],
+    "zk_moe_route_ext": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP],
+    "zk_moe_experts_ext": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _VP],
+    "zk_gate_rows": [_VP, _VP, _I, _I, _I, _VP],
+    "zk_cache_store": [_VP, _I, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_diff_attention_plain": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I,
+                                _F, _F, _F, _F, _I, _VP],
+    "zk_diff_join": [_VP, _VP, _I, _I, _I, _F, _F, _F, _VP],
     "zk_selective_scan": [_VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I,
                           _I, _I, _I, _VP, _VP, _VP],
 }
@@ -222,6 +235,7 @@ BF16_KERNEL_SIGNATURES = {
                                  _F, _F, _I, _I, _VP, _SZ, _I, _I, _I, _VP],
     "zk_latent_attention_bf16": [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _SZ, _I, _I, _I, _I, _I, _I, _I, _I, _F, _VP],
     "zk_moe_experts_grouped": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP],
+    "zk_moe_experts_grouped_ext": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _VP],
 }
 
 
