@@ -1,0 +1,452 @@
+"""Rotalorn models through the engine against the plain implementation (tests/plain/rotalorn_plain.py):
+every way of cutting the work, batches, pages and state slots used again, keys far back, keys just
+inside and just outside a window, the pair table across the cuts, the first tokens, long decoding,
+and greedy generation through ``Engine.generate``.  Small configurations of the tests' own, random
+weights; where random weights would hide a fault the scores are made sharp."""
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from conftest import ROOT
+from gpu_util import chunked_steps, make_runner, mixed_steps, run_steps, tail_decode_steps, whole_steps
+from plain import rotalorn_plain as P
+from rotalorn_util import (CFG_A, CFG_B, CFG_C, attention_layer, config, dense, diff_layer, latent_layer, moe,
+                           random_weights, write_model)
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {"A": (CFG_A, 21), "B": (CFG_B, 22), "C": (CFG_C, 23)}
+LENGTHS = {"A": [70, 1, 45, 2, 90, 33, 58], "B": [40, 75, 3, 52, 21], "C": [30, 64, 17, 49, 5]}
+PAGE = {"A": 4, "B": 8, "C": 16}
+
+
+def tokens_of(vocab, n, seed):
+    return np.random.default_rng(seed).integers(0, vocab, n).tolist()
+
+
+class Logits(np.ndarray):
+    """Plain logits [T, vocab] that also know, per row, how close the routers' choices were."""
+    calm = None
+
+
+CLOSE_CALL = 0.02      # a gap between two experts' scores that bfloat16 rounding of the input may close
+
+
+def reference(cfg, w, tokens):
+    margins = []
+    z = P.forward(cfg, w, tokens, np.float64, margins=margins).view(Logits)
+    z.calm = np.min(np.stack(margins), axis=0) > CLOSE_CALL if margins else np.ones(len(z), bool)
+    return z
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name, (cfg, seed) in CONFIGS.items():
+        w = random_weights(cfg, seed)
+        streams = {f"r{i}": tokens_of(cfg["vocab"], n, 50 + i) for i, n in enumerate(LENGTHS[name])}
+        refs = {r: reference(cfg, w, t) for r, t in streams.items()}
+        for dtype in ("float32", "bfloat16"):
+            folder = write_model(str(tmp_path_factory.mktemp(f"rotalorn{name}_{dtype}")), cfg, w, dtype)
+            out[(name, dtype)] = (folder, streams, refs)
+    return out
+
+
+def assert_close(got, want, dtype, what=""):
+    """Against the float64 values, relative to the largest logit.  float32 differs by the order of
+    its sums alone.  bfloat16 rounds every product's inputs: nine rows in ten within 5 %, every row
+    within 30 %; a wrong key, window, pair or expert moves most rows by the logits' own size.  A
+    token whose choice of experts was a close call in the plain run may go to another expert in
+    bfloat16 (and so may the tokens behind it that read what it left in a cache): such rows
+    count among the nine in ten but are not held to the bound for every row."""
+    calm = getattr(want, "calm", None)
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    assert got.shape == want.shape, f"{what}: shape {got.shape} vs {want.shape}"
+    err = np.abs(got - want).reshape(len(want), -1).max(axis=1) / max(1.0, np.abs(want).max())
+    if dtype == "float32":
+        ok = err.max() <= 3e-5
+    else:
+        held = err if calm is None or len(calm) != len(err) else err[calm]
+        ok = (held.size == 0 or held.max() <= 0.30) and np.quantile(err, 0.9) <= 0.05
+    if not ok:
+        raise AssertionError(f"{what}: largest relative error {err.max():.3e} at row {int(np.argmax(err))}, "
+                             f"nine in ten below {np.quantile(err, 0.9):.3e}")
+
+
+def check(rows, refs, dtype, what):
+    assert set(rows) == set(refs)
+    for r in refs:
+        assert_close(rows[r], refs[r], dtype, f"{what} {r}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_every_split_matches_the_plain_implementation(models, name, dtype):
+    folder, streams, refs = models[(name, dtype)]
+    runner = make_runner(folder, dtype, page_size=PAGE[name], cache_tokens=128, max_seqs=2, max_batch_tokens=128,
+                         max_model_len=128)
+    whole = run_steps(runner, streams, whole_steps(streams))
+    check(whole, refs, dtype, "whole")
+    tail = run_steps(runner, streams, tail_decode_steps(streams, tail=40))
+    check(tail, refs, dtype, "last 40 one by one")
+    one = run_steps(runner, streams, tail_decode_steps(streams, tail=1000))
+    check(one, refs, dtype, "token by token")
+    chunk = run_steps(runner, streams, chunked_steps(streams))
+    check(chunk, refs, dtype, "portions")
+    pairs = run_steps(runner, streams, chunked_steps(streams, sizes=(2,)))
+    check(pairs, refs, dtype, "portions of two")
+    if dtype == "float32":
+        # every sum runs in an order fixed by positions and channels alone: the cuts change nothing
+        for r in streams:
+            for other in (tail, one, chunk, pairs):
+                assert np.array_equal(whole[r], other[r]), r
+    assert all(p.free_pages == p.num_pages for p in runner.manager.pools)
+    assert runner.manager.slots.free_slots == 2
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_batches_with_pages_and_slots_used_again(models, name, dtype):
+    folder, streams, refs = models[(name, dtype)]
+    page = PAGE[name]
+    pages_of = lambda n: -(-n // page)
+    room = sum(sorted((pages_of(len(t)) for t in streams.values()), reverse=True)[:3])
+    runner = make_runner(folder, dtype, page_size=page, num_pages=room, max_seqs=3, max_batch_tokens=128,
+                         max_model_len=128)
+    alone = run_steps(runner, streams, whole_steps(streams))
+    for seed in (0, 1):
+        steps = mixed_steps(streams, seed=seed, max_live=3, room=room, page=page, decode_tail=9)
+        assert any(any(n > 1 for _, n in e) and any(n == 1 for _, n in e) for e, _ in steps)
+        slots_seen = {}
+
+        def observe(_):
+            for r in runner.manager.live():
+                slots_seen.setdefault(runner.manager.slot(r), set()).add(r)
+
+        rows = run_steps(runner, streams, steps, observe)
+        check(rows, refs, dtype, f"mixed seed {seed}")
+        assert any(len(v) >= 2 for v in slots_seen.values()), "no state slot was used again"
+        if dtype == "float32":
+            for r in streams:
+                assert np.array_equal(rows[r], alone[r]), f"{r} differs from its run alone"
+    assert all(p.free_pages == p.num_pages for p in runner.manager.pools)
+
+
+# ---------------------------------------------------------------- keys far back, and a window's edge
+MARK = 49          # two tokens, MARK and MARK - 1, that stand only where a test puts them
+
+
+def one_layer(kind, window, sizes="small"):
+    """One layer of the given kind and nothing else that looks back (no pair table)."""
+    big = sizes == "big"          # sizes that the matrix-core kernels take in bfloat16
+    if kind == "attention":
+        return attention_layer(heads=2, kv_heads=1, dim=64 if big else 48, rot_dims=16 if big else 4, base=30.0,
+                               scaling=(4.0, 1.0, 8.0, 128), window=window)
+    if kind == "latent_attention":
+        C = 56 if big else 48
+        return latent_layer(heads=2, dim=16, rot_dim=8 if big else 4, vdim=24, kv_rank=C, q_rank=C, base=30.0, window=window)
+    return diff_layer(heads=2, kv_heads=1, dim=32 if big else 16, vdim=32 if big else 24, diff=0.3, softcap=30.0,
+                      q_temp=(0.3, 50))
+
+
+def round16(a):
+    from zse_amd.weights.safetensors import bf16_bits_to_f32, f32_to_bf16_bits
+    return bf16_bits_to_f32(f32_to_bf16_bits(np.asarray(a, np.float32)))
+
+
+def a_key_that_is_found(cfg, w):
+    """Random weights spread a softmax over hundreds of keys, and no single key matters.  Here the
+    one layer is taken apart so that one does: keys read the first half of the width and values
+    the second; queries are the keys' own projection (rotated channels emptied, so that distance
+    takes nothing off a score); and the tokens MARK and MARK - 1 share the first half of their
+    embeddings and differ in the second.  A query of the one then scores a key of the other about
+    as high as its own, far above every other key, and what it gets from there is another value."""
+    w = dict(w)
+    l = cfg["layers"][0]
+    mx, m, W = l["mixer"], "l0.mix.", cfg["width"]
+    H, D, half = mx["heads"], mx["dim"], cfg["width"] // 2
+    tidy = lambda v: (v - v.mean()) / np.sqrt(((v - v.mean()) ** 2).mean())
+    e = w["embed"].copy()
+    e[MARK, :half] = e[MARK - 1, :half] = tidy(e[MARK, :half])
+    e[MARK, half:] = tidy(e[MARK, half:])
+    e[MARK - 1, half:] = -e[MARK, half:]          # opposite second halves: rows of equal size, values that differ most
+    w["embed"] = round16(e)
+    nb = w["l0.norm1.b"].copy()
+    nb[half:] = 0.0
+    w["l0.norm1.b"] = nb
+    w[m + "o"] = round16(w[m + "o"] * 3.0)          # what the mixer says counts for more of the logits
+    if l["type"] == "attention":
+        G, R = mx["kv_heads"], mx["rot"]["dims"]
+        match, val = slice(R, D - D // 4), slice(D - D // 4, D)      # channels that are compared, channels that carry a value
+        k, kb = w[m + "k"].reshape(G, D, W).copy(), w[m + "k.b"].reshape(G, D).copy()
+        k[:, :D - D // 4, half:], k[:, val, :half], kb[:, val] = 0.0, 0.0, 0.0      # (the rotated channels read the first half too)
+        of = [h // (H // G) for h in range(H)]
+        q, qb = np.zeros((H, D, W), np.float32), np.zeros((H, D), np.float32)
+        q[:, match], qb[:, match] = k[of][:, match], kb[of][:, match]
+        w[m + "k"], w[m + "q"], w[m + "q.b"] = k.reshape(G * D, W), q.reshape(H * D, W), qb.reshape(H * D)
+        w[m + "k.b"] = kb.reshape(G * D)
+        w[m + "q.norm"], w[m + "k.norm"] = np.ones(H * D, np.float32), np.ones(G * D, np.float32)
+    elif l["type"] == "latent_attention":
+        R, C, E = mx["rot_dim"], mx["kv_rank"], mx["vdim"]
+        dkv = w[m + "dkv"].copy()
+        dkv[:C // 2, half:], dkv[C // 2:C, :half] = 0.0, 0.0
+        uk, uv = w[m + "uk"].reshape(H, D, C).copy(), w[m + "uv"].reshape(H, E, C).copy()
+        uk[:, :, C // 2:], uv[:, :, :C // 2] = 0.0, 0.0
+        dq = dkv[:C].copy()
+        dq[C // 2:] = 0.0
+        uq = np.zeros((H, D + R, C), np.float32)
+        uq[:, :D] = uk
+        w[m + "dkv"], w[m + "uk"], w[m + "uv"] = dkv, uk.reshape(H * D, C), uv.reshape(H * E, C)
+        w[m + "dq"], w[m + "dq.norm"], w[m + "uq"] = dq, w[m + "dkv.norm"].copy(), uq.reshape(H * (D + R), C)
+    else:
+        G = mx["kv_heads"]
+        k, v = w[m + "k"].reshape(G, 2 * D, W).copy(), w[m + "v"].copy()
+        k[:, :, half:], v[:, :half] = 0.0, 0.0
+        w[m + "k"], w[m + "v"] = k.reshape(G * 2 * D, W), v
+        w[m + "q"] = k[[h // (H // G) for h in range(H)]].reshape(H * 2 * D, W).copy()
+    return w
+
+
+def sharp_enough(cfg, w, base, other, row):
+    """The scale of the scores at which the one key matters most at the row looked at."""
+    best = None
+    for scale in (0.25, 0.5, 1.0, 2.0, 4.0, 8.0, 16.0):
+        cfg["layers"][0]["mixer"]["scale"] = scale
+        ref, ref_other = P.forward(cfg, w, base, np.float64), P.forward(cfg, w, other, np.float64)
+        effect = np.abs(ref_other[row] - ref[row]).max() / np.abs(ref[row]).max()
+        if best is None or effect > best[0]:
+            best = (effect, scale, ref, ref_other)
+    assert best[0] > 0.05, "the key does not matter at any scale in this draw"
+    cfg["layers"][0]["mixer"]["scale"] = best[1]
+    return best[2], best[3]
+
+
+def unmarked(n, seed):
+    return np.random.default_rng(seed).integers(0, MARK - 1, n).tolist()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kind,sizes", [("attention", "small"), ("attention", "big"), ("latent_attention", "small"),
+                                        ("latent_attention", "big"), ("attention_2", "small"), ("attention_2", "big")])
+def test_a_key_hundreds_of_tokens_back(tmp_path, kind, sizes, dtype):
+    cfg = config([one_layer(kind, None, sizes)], vocab=MARK + 1, width=32, bigram=None)
+    w = a_key_that_is_found(cfg, random_weights(cfg, 11))
+    n, far = 330, 17
+    base = unmarked(n, 21)
+    base[far], base[-1] = MARK, MARK - 1
+    other = list(base)
+    other[far] = 3
+    ref, ref_other = sharp_enough(cfg, w, base, other, -1)
+    folder = write_model(str(tmp_path / f"far_{kind}_{dtype}"), cfg, w, dtype)
+    runner = make_runner(folder, dtype, page_size=16, cache_tokens=2 * 384, max_seqs=2, max_batch_tokens=512, max_model_len=384)
+    streams = {"base": base, "other": other}
+    for how, steps in (("prompt", whole_steps(streams)), ("decoded", tail_decode_steps(streams, tail=20)),
+                       ("portions", chunked_steps(streams, sizes=(64, 3, 31, 2)))):
+        rows = run_steps(runner, streams, steps)
+        assert_close(rows["base"], ref, dtype, f"{how} base")
+        assert_close(rows["other"], ref_other, dtype, f"{how} other")
+        assert np.abs(rows["other"][-1] - rows["base"][-1]).max() > 0.025 * np.abs(ref[-1]).max(), how
+
+
+@pytest.mark.parametrize("kind,sizes", [("attention", "small"), ("attention", "big"), ("latent_attention", "small"),
+                                        ("latent_attention", "big")])
+@pytest.mark.parametrize("window,page", [(19, 4), (16, 16), (33, 8), (1, 4), (2, 16)])
+def test_keys_just_inside_and_just_outside_the_window(tmp_path, kind, sizes, window, page):
+    """One layer, no pair table: the logits at position p depend on the tokens p - window + 1 .. p
+    and on nothing else.  The key that the last token finds, put just outside the window, must not
+    move a single bit of the last row, in a prompt, in portions that end before, at and behind
+    the edge, and token by token; just inside it takes about half of the row's weight."""
+    cfg = config([one_layer(kind, window, sizes)], vocab=MARK + 1, width=32, bigram=None)
+    w = a_key_that_is_found(cfg, random_weights(cfg, 5))
+    n = 3 * window + 41
+    base = unmarked(n, 3)
+    p = n - 1
+    base[p] = MARK - 1
+    outside, inside = list(base), list(base)
+    outside[p - window] = MARK
+    if window > 1:
+        inside[p - window + 1] = MARK
+        sharp_enough(cfg, w, base, inside, p)
+    refs = {"base": P.forward(cfg, w, base, np.float64), "outside": P.forward(cfg, w, outside, np.float64),
+            "inside": P.forward(cfg, w, inside, np.float64)}
+    assert np.abs(refs["outside"][p] - refs["base"][p]).max() < 1e-12
+    streams = {"base": base, "outside": outside, "inside": inside}
+    for dtype in ("float32", "bfloat16"):
+        folder = write_model(str(tmp_path / f"edge_{dtype}"), cfg, w, dtype)
+        runner = make_runner(folder, dtype, page_size=page, cache_tokens=3 * 256, max_seqs=3, max_batch_tokens=256,
+                             max_model_len=256)
+        edge = p - window
+        ways = {"prompt": whole_steps(streams), "decoded": tail_decode_steps(streams, tail=window + 9),
+                "portions to the edge": chunked_steps(streams, sizes=(edge, 2, 5)),
+                "portions over the edge": chunked_steps(streams, sizes=(edge - 1, 3, 2, 7)),
+                "portions behind the edge": chunked_steps(streams, sizes=(edge + 1, 2)),
+                "portions of two": chunked_steps(streams, sizes=(2,))}
+        for how, steps in ways.items():
+            rows = run_steps(runner, streams, steps)
+            for r in streams:
+                assert_close(rows[r], refs[r], dtype, f"{how} {r}")
+            if dtype == "float32":
+                assert np.array_equal(rows["outside"][p], rows["base"][p]), f"{how}: a key outside the window was seen"
+            if window > 1:
+                assert np.abs(rows["inside"][p] - rows["base"][p]).max() > 0.025 * np.abs(refs["base"][p]).max(), \
+                    f"{how}: a key inside the window was lost"
+
+
+# ---------------------------------------------------------------- the pair table
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_pair_table_across_cuts_and_slots(tmp_path, dtype):
+    """A pair table that outweighs the embedding, and no mixer weight to speak of: a wrong previous
+    token (a stale one of the slot's last owner, none at the start of a portion, a hash of other
+    multipliers) moves the logits by their own size."""
+    cfg = config([attention_layer(heads=1, kv_heads=1, dim=8, rot_dims=8, window=4, mlp=dense(16))], vocab=40, width=16,
+                 bigram=(23, 5, 11))
+    w = random_weights(cfg, 8)
+    w["bigram"] = (w["bigram"] * 6.0).astype(np.float32)
+    streams = {f"r{i}": tokens_of(cfg["vocab"], n, 70 + i) for i, n in enumerate([25, 1, 14, 2, 31])}
+    refs = {r: P.forward(cfg, w, t, np.float64) for r, t in streams.items()}
+    first_row_only = dict(w)
+    first_row_only["bigram"] = np.repeat(w["bigram"][-1:], len(w["bigram"]), axis=0)
+    assert np.abs(P.forward(cfg, first_row_only, streams["r0"], np.float64) - refs["r0"])[1:].max() > 0.3 * np.abs(refs["r0"]).max()
+    folder = write_model(str(tmp_path / f"pairs_{dtype}"), cfg, w, dtype)
+    runner = make_runner(folder, dtype, page_size=4, cache_tokens=64, max_seqs=1, max_batch_tokens=64, max_model_len=64)
+    # one slot, one request after the other, each cut differently
+    for sizes in ((1000,), (1,), (2,), (3, 1, 1, 6), (7, 2)):
+        for r in streams:
+            rows = run_steps(runner, {r: streams[r]}, chunked_steps({r: streams[r]}, sizes=sizes))
+            assert_close(rows[r], refs[r], dtype, f"{r} in portions of {sizes}")
+    # several requests in one step, some with one token
+    runner = make_runner(folder, dtype, page_size=4, num_pages=24, max_seqs=3, max_batch_tokens=64, max_model_len=64)
+    for seed in (0, 1, 2):
+        rows = run_steps(runner, streams, mixed_steps(streams, seed=seed, max_live=3, room=24, page=4, decode_tail=5))
+        for r in streams:
+            assert_close(rows[r], refs[r], dtype, f"mixed {seed} {r}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_shared_experts_gate_and_the_scores_on_the_outputs(tmp_path, dtype):
+    """Routed experts that outweigh the rest: scores on the inputs, renormalised scores or a shared
+    expert without its gate would move every logit."""
+    cfg = config([diff_layer(heads=1, kv_heads=1, dim=8, vdim=8, mlp=moe(6, 2, 16, 24))], vocab=60, width=32)
+    w = random_weights(cfg, 31)
+    w["l0.mlp.shared.sg"] = (w["l0.mlp.shared.sg"] * 8.0).astype(np.float32)
+    toks = tokens_of(cfg["vocab"], 40, 5)
+    ref = reference(cfg, w, toks)
+    ungated = dict(w)
+    ungated["l0.mlp.shared.sg"] = np.zeros_like(w["l0.mlp.shared.sg"])
+    assert np.abs(P.forward(cfg, ungated, toks, np.float64) - ref).max() > 0.05 * np.abs(ref).max()
+    folder = write_model(str(tmp_path / f"moe_{dtype}"), cfg, w, dtype)
+    runner = make_runner(folder, dtype, page_size=8, cache_tokens=128, max_seqs=1, max_batch_tokens=64, max_model_len=64)
+    for steps in (whole_steps({"r": toks}), tail_decode_steps({"r": toks}, tail=30), chunked_steps({"r": toks})):
+        assert_close(run_steps(runner, {"r": toks}, steps)["r"], ref, dtype, "experts")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_through_every_kind_of_layer(models, dtype):
+    cfg, seed = CONFIGS["A"]
+    folder = models[("A", dtype)][0]
+    w = random_weights(cfg, seed)
+    toks = tokens_of(cfg["vocab"], 240, 77)
+    ref = reference(cfg, w, toks)
+    runner = make_runner(folder, dtype, page_size=4, cache_tokens=256, max_seqs=1, max_batch_tokens=64, max_model_len=256)
+    rows = run_steps(runner, {"r": toks}, tail_decode_steps({"r": toks}, tail=230))
+    assert_close(rows["r"], ref, dtype, "230 tokens one by one")
+
+
+def test_the_first_tokens_of_a_sequence(models):
+    """Positions 0 to 3: the pair table's row of its own, windows larger than what there is, a
+    temperature that has not changed yet."""
+    for name in ("A", "B", "C"):
+        cfg, seed = CONFIGS[name]
+        folder = models[(name, "float32")][0]
+        w = random_weights(cfg, seed)
+        runner = make_runner(folder, "float32", page_size=4, cache_tokens=64, max_seqs=2, max_batch_tokens=64, max_model_len=64)
+        for n in (1, 2, 3, 4):
+            toks = tokens_of(cfg["vocab"], n, 200 + n)
+            ref = P.forward(cfg, w, toks, np.float64)
+            for steps in (whole_steps({"r": toks}), tail_decode_steps({"r": toks}, tail=10)):
+                rows = run_steps(runner, {"r": toks}, steps)
+                assert_close(rows["r"], ref, "float32", f"{name}: {n} tokens")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_slot_taken_over_starts_from_zero(models, dtype):
+    """One slot, requests one after the other: none must see the token the one before left there."""
+    folder, streams, refs = models[("A", dtype)]
+    runner = make_runner(folder, dtype, page_size=4, cache_tokens=128, max_seqs=1, max_batch_tokens=128, max_model_len=128)
+    for r in ("r0", "r4", "r2", "r0"):
+        rows = run_steps(runner, {r: streams[r]}, chunked_steps({r: streams[r]}, sizes=(9, 1, 4)))
+        assert_close(rows[r], refs[r], dtype, r)
+
+
+# ---------------------------------------------------------------- the engine's own entry point
+def plain_greedy(cfg, w, prompt, n):
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(np.argmax(P.forward(cfg, w, toks, np.float64)[-1])))
+    return toks[len(prompt):]
+
+
+def test_greedy_generation_through_the_engine(models):
+    from zse_amd.engine.engine import Engine
+    from zse_amd.sampling.sampler import SamplingParams
+    cfg, seed = CONFIGS["A"]
+    folder = models[("A", "float32")][0]
+    w = random_weights(cfg, seed)
+    prompts = [tokens_of(cfg["vocab"], n, 300 + n) for n in (5, 23, 1, 40, 12, 31)]
+    want = [plain_greedy(cfg, w, p, 12) for p in prompts]
+    # four places for six requests, portions of 16: prompts are cut, requests wait for a slot
+    with Engine(folder, dtype="float32", block_size=4, num_blocks=64, max_batch_tokens=32, max_batch_seqs=4,
+                prefill_chunk_size=16, max_seq_len=128) as eng:
+        got = eng.generate(prompts, SamplingParams(max_tokens=12, temperature=0.0))
+        assert got == want
+        again = eng.generate(prompts[:2], SamplingParams(max_tokens=12, temperature=0.0))
+        assert again == want[:2]
+    with Engine(folder, dtype="float32", block_size=4, num_blocks=64, max_batch_tokens=32, max_batch_seqs=4,
+                prefill_chunk_size=16, max_seq_len=128, use_graphs=False) as eng:
+        assert eng.generate(prompts, SamplingParams(max_tokens=12, temperature=0.0)) == want
+
+
+def test_generation_in_bfloat16_through_graphs_does_not_depend_on_the_company(models):
+    from zse_amd.engine.engine import Engine
+    from zse_amd.sampling.sampler import SamplingParams
+    cfg, _ = CONFIGS["A"]
+    folder = models[("A", "bfloat16")][0]
+    prompts = [tokens_of(cfg["vocab"], n, 400 + n) for n in (9, 30, 17)]
+    sp = SamplingParams(max_tokens=10, temperature=0.0)
+    with Engine(folder, dtype="bfloat16", block_size=8, num_blocks=64, max_batch_tokens=64, max_batch_seqs=4,
+                prefill_chunk_size=64, max_seq_len=128) as eng:
+        together = eng.generate(prompts, sp)
+        alone = [eng.generate([p], sp)[0] for p in prompts]
+        assert eng.runner.graph_runs > 0, "no decode step was replayed from a graph"
+    assert together == alone
+    with Engine(folder, dtype="bfloat16", block_size=8, num_blocks=64, max_batch_tokens=64, max_batch_seqs=4,
+                prefill_chunk_size=64, max_seq_len=128, use_graphs=False) as eng:
+        assert eng.generate(prompts, sp) == together
+
+
+def test_the_trace_program_serves_the_design(models, tmp_path):
+    cfg, seed = CONFIGS["A"]
+    folder, streams, refs = models[("A", "float32")]
+    out = tmp_path / "out"
+    a, b = streams["r0"], streams["r2"]
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:7], "want": [0, 6]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[7:9], "want": []}, {"id": "b", "tokens": b[:40], "want": [39]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[40:41], "want": [0]}, {"id": "a", "tokens": a[9:], "want": [len(a) - 10]}],
+         "end": ["a"]},
+        {"step": 3, "entries": [{"id": "b", "tokens": b[41:], "want": [len(b) - 42]}], "end": ["b"]},
+    ]
+    p = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", str(out),
+                        "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                       capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    V = cfg["vocab"]
+    read = lambda i: np.fromfile(str(out / f"{i}.f32"), dtype="<f4").reshape(-1, V)
+    assert_close(read(0), refs["r0"][[0, 6]], "float32", "step 0")
+    assert_close(read(1), refs["r2"][[39]], "float32", "step 1")
+    assert_close(read(2), np.stack([refs["r2"][40], refs["r0"][len(a) - 1]]), "float32", "step 2")
+    assert_close(read(3), refs["r2"][[len(b) - 1]], "float32", "step 3")

@@ -111,6 +111,18 @@ class RotalornConfig:
         return RotalornMLP("moe", ff, experts, top, sff)
 
     @staticmethod
+    def _scaling(rot: Optional[dict], q: Problems):
+        sc = need(rot, "scaling", dict, q, default=None, allow_none=True) if rot is not None else None
+        if sc is None:
+            return None
+        vals = [need(sc, key, float, q, required=True) for key in ("factor", "low", "high", "original")]
+        if None in vals:
+            return None
+        q.require(vals[0] > 0 and vals[3] > 0 and 0 < vals[1] < vals[2],
+                  f"rot.scaling: factor and original positive and 0 < low < high, got {vals}")
+        return tuple(vals)
+
+    @staticmethod
     def _window(mx: dict, q: Problems) -> Optional[int]:
         mask = need(mx, "mask", dict, q, default=None, allow_none=True)
         if mask is None:
@@ -164,14 +176,7 @@ class RotalornConfig:
                 rot = need(mx, "rot", dict, q, default=None, allow_none=True)
                 base = need(rot, "base", float, q, required=True) if rot is not None else None
                 dims = need(rot, "dims", int, q, default=dim) if rot is not None else 0
-                sc = need(rot, "scaling", dict, q, default=None, allow_none=True) if rot is not None else None
-                scaling = None
-                if sc is not None:
-                    vals = [need(sc, key, float, q, required=True) for key in ("factor", "low", "high", "original")]
-                    if None not in vals:
-                        q.require(vals[0] > 0 and vals[3] > 0 and 0 < vals[1] < vals[2],
-                                  f"rot.scaling: factor and original positive and 0 < low < high, got {vals}")
-                        scaling = tuple(vals)
+                scaling = RotalornConfig._scaling(rot, q)
                 if not q.items:
                     q.require(kvh > 0 and heads % kvh == 0, f"heads ({heads}) must be a multiple of kv_heads ({kvh})")
                     q.require(rot is None or (base > 0 and base != 1 and dims % 2 == 0 and 0 < dims <= dim),
@@ -187,6 +192,7 @@ class RotalornConfig:
                 rot = need(mx, "rot", dict, q, required=True) or {}
                 base = need(rot, "base", float, q, required=True)
                 dims = need(rot, "dims", int, q, default=rdim)
+                scaling = RotalornConfig._scaling(rot, q)
                 if not q.items:
                     q.require(rdim > 0 and rdim % 2 == 0 and rank > 0 and qrank > 0,
                               f"rot_dim must be even and positive, kv_rank and q_rank positive, got {rdim}, {rank}, {qrank}")
@@ -194,7 +200,8 @@ class RotalornConfig:
                     q.require(base > 0 and base != 1, f"rot.base must be positive, got {base}")
                     q.require(rank + rdim <= 1024, f"kv_rank + rot_dim up to 1024, got {rank + rdim}")
                 layers.append(RotalornLayer("latent_attention", heads, dim, vdim, mlp, scale=scale, window=window,
-                                            rot_base=base, rot_dim=rdim or 0, kv_rank=rank or 0, q_rank=qrank or 0))
+                                            rot_base=base, rot_dim=rdim or 0, kv_rank=rank or 0, q_rank=qrank or 0,
+                                            rot_scaling=scaling))
             elif typ == "attention_2":
                 kvh = need(mx, "kv_heads", int, q, default=heads)
                 diff = need(mx, "diff", float, q, required=True)
@@ -238,7 +245,8 @@ def rotalorn_plan(c: RotalornConfig) -> ModelPlan:
             mixer = LatentAttentionSpec(
                 hidden_size=c.width, num_heads=l.heads, head_dim=l.dim, rotary_dim=l.rot_dim, value_dim=l.vdim,
                 latent_dim=l.kv_rank, scale=l.scale, eps=c.eps,
-                position=RotarySpec(head_dim=l.rot_dim, rotary_dim=l.rot_dim, theta=l.rot_base),
+                position=RotarySpec(head_dim=l.rot_dim, rotary_dim=l.rot_dim, theta=l.rot_base,
+                                    wavelength_scaling=l.rot_scaling),
                 names={"q": mix + "uq", "q_down": mix + "dq", "q_down_norm": mix + "dq.norm", "down": mix + "dkv",
                        "down_norm": mix + "dkv.norm", "up_k": mix + "uk", "up_v": mix + "uv", "gate": mix + "g",
                        "o": mix + "o"},
