@@ -492,6 +492,33 @@ def bumolix_config(width, heads, kv_heads, dim, ff, groups, vocab, window):
             "layers": layers}
 
 
+def rotalorn_config(width, heads, kv_heads, dim, ff, groups, vocab, window):
+    """``groups`` times (differential attention, attention whose values are its keys, latent attention with
+    queries through a latent), each with the relative's feed-forward: eight routed experts of a quarter of
+    the feed-forward size, two a token, and a shared expert of half of it.  The attention has the
+    relative's heads and a window; the differential attention has as many heads with two maps of
+    ``dim`` channels over values of ``dim`` (twice the query and key rows of the attention beside it);
+    the latent attention has the relative's sizes, a query latent of half the width and the window."""
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2}, "shared": {"ff": ff // 2}}
+    layers = []
+    for _ in range(groups):
+        layers += [
+            {"type": "attention_2", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                              "diff": 0.5, "softcap": 30.0, "q_temp": {"coef": 0.1, "every": 1024}},
+             "mlp": dict(moe)},
+            {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                            "mask": {"size": window},
+                                            "rot": {"base": 10000.0, "dims": dim // 2,
+                                                    "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 2048}}},
+             "mlp": dict(moe)},
+            {"type": "latent_attention", "mixer": {"heads": heads, "dim": dim // 2, "rot_dim": dim // 4, "vdim": dim // 2,
+                                                   "kv_rank": 2 * dim, "q_rank": width // 2, "scale": (3 * dim // 4) ** -0.5,
+                                                   "mask": {"size": window}, "rot": {"base": 10000.0, "dims": dim // 4}},
+             "mlp": dict(moe)}]
+    return {"architecture": "Rotalorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}}, "layers": layers}
+
+
 # what is timed, beside which relative, against which plain implementation it is checked first, and
 # the deviations of the random tensors that are not drawn like matrices or gains
 DESIGNS = {
@@ -501,6 +528,10 @@ DESIGNS = {
                     std_of={".conv": 0.3, "A_log": 0.5, "dt_bias": 0.5, "mix.norm": 1.0, "dkv.norm": 1.0, ".sink": 1.0, ".b": 0.02,
                             "router": 0.1},
                     beside=("dafotar", "Dafotar", dafotar_config)),
+    "rotalorn": dict(name="Rotalorn", make=rotalorn_config, plain="rotalorn_plain",
+                     std_of={".b": 0.02, "router": 0.1, ".lq1": 0.3, ".lk1": 0.3, ".lq2": 0.3, ".lk2": 0.3, ".norm": 1.0,
+                             "norm1": 1.0, "final.norm": 1.0, ".sg": 0.1, "bigram": 0.02},
+                     beside=("pubunex", "Pubunex", pubunex_config)),
     "bumolix": dict(name="Bumolix", make=bumolix_config, plain="bumolix_plain",
                     std_of={".b": 0.02, ".conv": 0.3, "A_log": 0.5, "dt.b": 0.5, "a2.b": 1.0, ".D": 0.5, "norm": 0.5},
                     beside=("dafotar", "Dafotar", dafotar_config)),
@@ -639,7 +670,7 @@ def main():
                     help="instead of the default workload: prefill and decode of this design beside its closest relative "
                          "(Dafotar beside Gemma 2, Pubunex and Bumolix beside Dafotar) at equal layer sizes")
     ap.add_argument("--design-sizes", default="w1024,w2048,w4096", help="with --design: which of " + ", ".join(DESIGN_SIZES))
-    ap.add_argument("--only-model", choices=["bumolix", "dafotar", "gemma2", "pubunex"], default=None, help="with --design, a profiling aid: one of the two")
+    ap.add_argument("--only-model", choices=["bumolix", "dafotar", "gemma2", "pubunex", "rotalorn"], default=None, help="with --design, a profiling aid: one of the two")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)

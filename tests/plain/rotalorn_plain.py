@@ -221,13 +221,13 @@ def gated(x, w, pre, act, dt):
 def route(x, w_router, top, dt):
     """softmax over all experts of the router's logits; the ``top`` largest (the lower index among
     equals), their scores as weights, not renormalised.  Returns ids [T, top], weights [T, top]
-    and each token's margin between the last chosen and the first left-out score."""
+    and each token's margin between the logits of the last chosen and the first left-out expert."""
     z = x.astype(np.float32).astype(dt) @ w_router.astype(dt).T
     s = np.exp(z - z.max(axis=1, keepdims=True))
     s = s / s.sum(axis=1, keepdims=True)
     order = np.argsort(-s, axis=1, kind="stable")
     ids = order[:, :top]
-    srt = np.take_along_axis(s, order, axis=1)
+    srt = np.take_along_axis(z, order, axis=1)              # the margin is taken between logits
     margin = srt[:, top - 1] - srt[:, top] if s.shape[1] > top else np.full(len(s), np.inf)
     return ids, np.take_along_axis(s, ids, axis=1), margin
 

@@ -32,7 +32,7 @@ class Logits(np.ndarray):
     calm = None
 
 
-CLOSE_CALL = 0.02      # a gap between two experts' scores that bfloat16 rounding of the input may close
+CLOSE_CALL = 0.1       # a gap between two experts' router logits that bfloat16 rounding of the input may close
 
 
 def reference(cfg, w, tokens):

@@ -169,7 +169,7 @@ def test_differential_attention_over_pages(dev, H, G, D, E, window, cap, temp):
     kk = {r: rng.normal(size=(n, G, 2, D)).astype(np.float32) for r, n in enumerate(lens)}
     v = {r: rng.normal(size=(n, G, E)).astype(np.float32) for r, n in enumerate(lens)}
     table, slot_of, pages = paged(rt, rng, lens, bs)
-    kc, vc = rt.zeros((pages, G, bs, 2 * D), "float32"), rt.zeros((pages, G, bs, E), "float32")
+    kc, vc = rt.zeros((pages, 2 * G, bs, D), "float32"), rt.zeros((pages, G, bs, E), "float32")
     ld = (H + G) * 2 * D + G * E + 3
 
     def rows_of(r, lo, hi):
@@ -188,7 +188,7 @@ def test_differential_attention_over_pages(dev, H, G, D, E, window, cap, temp):
                 slots += [slot_of(r, j) for j in range(lo, hi)]
         x = f32(rt, np.concatenate(rows))
         T = len(pos)
-        k.zk_cache_store(x.ptr, ld, H * 2 * D, (H + G) * 2 * D, i32(rt, slots).ptr, kc.ptr, vc.ptr, T, G, 2 * D, E, bs, 0, rt.stream)
+        k.zk_cache_store(x.ptr, ld, H * 2 * D, (H + G) * 2 * D, i32(rt, slots).ptr, kc.ptr, vc.ptr, T, 2 * G, D, G, E, bs, 0, rt.stream)
     out = rt.empty((T, H * E), "float32")
     k.zk_diff_attention_plain(x.ptr, ld, kc.ptr, vc.ptr, i32(rt, table).ptr, table.shape[1], i32(rt, req).ptr, i32(rt, pos).ptr,
                               out.ptr, T, H, G, D, E, bs, scale, cap, window, 0, lam, diff, eps,

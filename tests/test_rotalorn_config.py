@@ -39,9 +39,9 @@ def test_what_a_request_keeps():
     assert all(isinstance(n, PagedKV) for n in needs)
     latent, diff, attn, diff2 = needs
     assert (latent.num_kv_heads, latent.head_dim, latent.window, latent.values_in_keys) == (1, 24, 13, True)
-    assert (diff.num_kv_heads, diff.head_dim, diff.value_dim, diff.window) == (2, 24, 24, None)     # both maps' keys side by side
+    assert (diff.num_kv_heads, diff.head_dim, diff.value_heads, diff.value_dim, diff.window) == (4, 12, 2, 24, None)   # a key head a map
     assert (attn.num_kv_heads, attn.head_dim, attn.window) == (2, 24, 21)
-    assert (diff2.head_dim, diff2.value_dim) == (16, 8)
+    assert (diff2.num_kv_heads, diff2.head_dim, diff2.value_heads, diff2.value_dim) == (4, 8, 2, 8)
     assert m.embedding.state_bytes() == 4                     # the previous token
     assert model_of(CFG_B).embedding.state_bytes() == 0       # no pair table, nothing kept
     assert model_of(CFG_B).cache_needs()[1].window is None and model_of(CFG_B).cache_needs()[3].window is None

@@ -52,7 +52,8 @@ struct AttnParams {
   const __bf16* q;
   int q_stride;
   const __bf16* kcache;   // [page][nkv][bs][hd]
-  const __bf16* vcache;   // [page][nkv][hd][bs]
+  const __bf16* vcache;   // [page][nkv >> v_shift][hd][bs]
+  int v_shift;            // 2^v_shift neighbouring key heads share one value head (0: a value head per key head)
   const int* block_table;
   int max_blocks;
   const int* q_start;     // [R + 1]
@@ -78,6 +79,14 @@ struct AttnParams {
   int wide_weights;       // 1: a weight meets the values as two bf16 numbers, its rounded value and what the
                           // rounding left (16 bits of mantissa instead of 8; one more product a tile)
 };
+
+// The query head that is the hq-th of key head kvh.  Without shared values: kvh * g + hq.  With
+// 2^v_shift maps of keys over one value head, key head (v, m) serves map m of the g query heads
+// of value head v, and a query head's maps lie side by side: ((v * g + hq) << v_shift) + m.
+__device__ __forceinline__ int q_head_of(const AttnParams& p, int kvh, int hq) {
+  const int g = p.nh / p.nkv;
+  return (((kvh >> p.v_shift) * g + hq) << p.v_shift) | (kvh & ((1 << p.v_shift) - 1));
+}
 
 // The first key a row at position ``pos`` sees.  It never decreases as pos grows, which is all
 // the kernels' bounds over groups and blocks of rows rest on.
@@ -172,7 +181,7 @@ __global__ __launch_bounds__(256, (HD16 <= 8 && !PAIR) ? 2 : 1) void attn_mfma_k
   const bool row_ok = tok < ntok;
   const int trow = qs + t0 + (row_ok ? tok : 0);
   const int pos = start + t0 + (row_ok ? tok : 0);
-  const int head = kvh * g + (row_ok ? hq : 0);
+  const int head = q_head_of(p, kvh, row_ok ? hq : 0);
   const int pos_lo = start + t0, pos_hi = start + t0 + ntok - 1;
   int key_lo = first_key(p, pos_lo);
   int key_hi = pos_hi;
@@ -246,8 +255,8 @@ __global__ __launch_bounds__(256, (HD16 <= 8 && !PAIR) ? 2 : 1) void attn_mfma_k
     for (int h = 0; h < 2; h++) {
       const int ka = min(key0 + h * 16 + 4 * lk, key_hi & ~3), kb = min(key0 + h * 16 + 8 + 4 * lk, key_hi & ~3);
       const int pa = max(pg.va[h], 0), pb = max(pg.vb[h], 0);
-      const __bf16* vpa = p.vcache + ((((size_t)pa * nkv + kvh) * hd) << bsh) + (ka & bmask);
-      const __bf16* vpb = p.vcache + ((((size_t)pb * nkv + kvh) * hd) << bsh) + (kb & bmask);
+      const __bf16* vpa = p.vcache + ((((size_t)pa * (nkv >> p.v_shift) + (kvh >> p.v_shift)) * hd) << bsh) + (ka & bmask);
+      const __bf16* vpb = p.vcache + ((((size_t)pb * (nkv >> p.v_shift) + (kvh >> p.v_shift)) * hd) << bsh) + (kb & bmask);
 #pragma unroll
       for (int dt = 0; dt < DT; dt++) {
         const bf16x4 va = *(const bf16x4*)(vpa + vrow[dt]);
@@ -483,7 +492,7 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
   const bool row_ok = tok < ntok;
   const int trow = qs + (row_ok ? t0 + tok : 0);
   const int pos = start + (row_ok ? t0 + tok : 0);
-  const int head = kvh * g + (row_ok ? hq : 0);
+  const int head = q_head_of(p, kvh, row_ok ? hq : 0);
   const int pos_lo = start + t0, pos_hi = start + t0 + ntok - 1;          // ntok == 0: no keys at all
   const int row_lo = first_key(p, pos);
   const int all_hi = ntok * g == 32 ? pos_lo : -1;
@@ -534,13 +543,14 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
     k_off[j] = (unsigned)(((kvh << bsh) + (kk & bmask)) * HD + col);
     k_lds[j] = kk * KLD + col;
     v_idx[j] = vk >> bsh;
-    v_off[j] = (unsigned)(((kvh * HD + d) << bsh) + (vk & bmask));
+    v_off[j] = (unsigned)((((kvh >> p.v_shift) * HD + d) << bsh) + (vk & bmask));
     // keys 8c + (0..3) go to piece 2h of the channel, keys 8c + 4 + (0..3) to piece 2h + 1,
     // both at slot 4 (c % 2), with h = c / 2
     const int c = vk >> 3;
     v_lds[j] = d * VLD + (c >> 1) * 16 + (c & 1) * 4;
   }
-  const size_t page_elems = ((size_t)nkv * HD) << bsh;        // of a page of K, and of a page of V
+  const size_t page_elems = ((size_t)nkv * HD) << bsh;        // of a page of K
+  const size_t v_page_elems = ((size_t)(nkv >> p.v_shift) * HD) << bsh;
   const int last_entry = p.max_blocks - 1;
   struct Pages { int k[PPT], v[PPT]; };
   struct Stage { bf16x8 k[PPT], v[PPT]; };
@@ -562,7 +572,7 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
 #pragma unroll
     for (int j = 0; j < PPT; j++) {
       st.k[j] = *(const bf16x8*)(p.kcache + ((size_t)max(pg.k[j], 0) * page_elems + (k_off[j] + in_page * HD)));
-      st.v[j] = *(const bf16x8*)(p.vcache + ((size_t)max(pg.v[j], 0) * page_elems + (v_off[j] + in_page)));
+      st.v[j] = *(const bf16x8*)(p.vcache + ((size_t)max(pg.v[j], 0) * v_page_elems + (v_off[j] + in_page)));
     }
   };
   auto stash = [&](int buf, const Stage& st) {
@@ -766,7 +776,7 @@ __global__ __launch_bounds__(64) void attn_portion_join_kernel(AttnParams p, int
     for (int j = 0; j < 4; j++) acc[j] += w * po[j * 64];
   }
   const float inv = 1.f / (l + sink_weight(p, m));
-  __bf16* orow = p.out + ((size_t)(qs + t0 + tok) * p.nh + kvh * g + hq) * p.hd;
+  __bf16* orow = p.out + ((size_t)(qs + t0 + tok) * p.nh + q_head_of(p, kvh, hq)) * p.hd;
 #pragma unroll
   for (int j = 0; j < 4; j++) {
     const int d = dt * 32 + 8 * j + 4 * lk;
@@ -825,7 +835,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const bool active = key_lo <= key_hi;          // a wave without keys still meets the others at the barrier
   const int g = p.nh / p.nkv;
   const bool col_ok = col < g;
-  const int head = kvh * g + (col_ok ? col : 0);
+  const int head = q_head_of(p, kvh, col_ok ? col : 0);
   const int trow = p.q_start[r];
 
   // the query operand waits in LDS (one 16-byte piece per lane and step), not in registers
@@ -864,8 +874,8 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     {
       const int ka = key0 + 4 * kq, kb = key0 + 16 + 4 * kq;
       const int pa = max(vpage[i][0], 0), pb = max(vpage[i][1], 0);
-      const __bf16* va_base = p.vcache + ((((size_t)pa * nkv + kvh) * hd) << bsh) + (ka & bmask);
-      const __bf16* vb_base = p.vcache + ((((size_t)pb * nkv + kvh) * hd) << bsh) + (kb & bmask);
+      const __bf16* va_base = p.vcache + ((((size_t)pa * (nkv >> p.v_shift) + (kvh >> p.v_shift)) * hd) << bsh) + (ka & bmask);
+      const __bf16* vb_base = p.vcache + ((((size_t)pb * (nkv >> p.v_shift) + (kvh >> p.v_shift)) * hd) << bsh) + (kb & bmask);
 #pragma unroll
       for (int dt = 0; dt < DT; dt++) {
         const int d = dt * 16 + col;
@@ -959,7 +969,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
       acc += e * sm_o[((size_t)w * g + c) * hd + d];
       l += e * sm_ml[(w * 16 + c) * 2 + 1];
     }
-    const size_t slot = ((size_t)(r - p.r_begin) * p.nh + kvh * g + c) * p.nchunks + block_x;
+    const size_t slot = ((size_t)(r - p.r_begin) * p.nh + q_head_of(p, kvh, c)) * p.nchunks + block_x;
     p.part_o[slot * hd + d] = acc;
     if (d == 0) {
       p.part_ml[slot * 2] = m;
@@ -1180,12 +1190,15 @@ long long zk_attention_bf16_max_context(int nh, int nkv, int hd, int decode_chun
 // mask_chunk > 0: a row sees the keys of its own chunk of that many positions (counted from
 // position 0) instead of a window; sink: a key of score 0 without a value in every denominator;
 // wide_weights: the weights keep 16 bits of mantissa in the product with the values.
-int zk_attention_bf16_masked(const void* q, int q_stride, const void* kcache, const void* vcache_t,
-                             const int* block_table, int max_blocks, const int* q_start, const int* ctx_len,
-                             void* out, int R, int r_prefill, int max_q_len, int max_ctx, int nh, int nkv,
-                             int hd, int bs, float scale, float softcap, int window, int decode_chunk,
-                             void* workspace, size_t workspace_bytes, int mask_chunk, int sink, int wide_weights,
-                             void* stream) {
+// v_shift: 2^v_shift neighbouring key heads read the values of one value head (the value cache
+// then holds nkv >> v_shift heads): several maps of keys over the same values.
+int zk_attention_bf16_maps(const void* q, int q_stride, const void* kcache, const void* vcache_t,
+                           const int* block_table, int max_blocks, const int* q_start, const int* ctx_len,
+                           void* out, int R, int r_prefill, int max_q_len, int max_ctx, int nh, int nkv,
+                           int hd, int bs, float scale, float softcap, int window, int decode_chunk,
+                           void* workspace, size_t workspace_bytes, int mask_chunk, int sink, int wide_weights,
+                           int v_shift, void* stream) {
+  ZK_REQUIRE(v_shift >= 0 && v_shift <= 4 && nkv % (1 << v_shift) == 0, "zk_attention_bf16: key heads in whole groups of a value head");
   ZK_REQUIRE(mask_chunk >= 0 && (mask_chunk == 0 || window == 0), "zk_attention_bf16: a window or a chunk, not both");
   ZK_REQUIRE(R >= 0 && r_prefill >= 0 && r_prefill <= R, "zk_attention_bf16: bad request counts");
   ZK_REQUIRE(zk_attention_bf16_supports(nh, nkv, hd, bs), "zk_attention_bf16: sizes not supported "
@@ -1208,7 +1221,7 @@ int zk_attention_bf16_masked(const void* q, int q_stride, const void* kcache, co
   hipStream_t s = (hipStream_t)stream;
   AttnParams p;
   p.q = (const __bf16*)q; p.q_stride = q_stride;
-  p.kcache = (const __bf16*)kcache; p.vcache = (const __bf16*)vcache_t;
+  p.kcache = (const __bf16*)kcache; p.vcache = (const __bf16*)vcache_t; p.v_shift = v_shift;
   p.block_table = block_table; p.max_blocks = max_blocks;
   p.q_start = q_start; p.ctx_len = ctx_len; p.out = (__bf16*)out;
   p.nh = nh; p.nkv = nkv; p.hd = hd; p.bs = bs;
@@ -1337,6 +1350,17 @@ int zk_attention_bf16_masked(const void* q, int q_stride, const void* kcache, co
   return 0;
 }
 
+int zk_attention_bf16_masked(const void* q, int q_stride, const void* kcache, const void* vcache_t,
+                             const int* block_table, int max_blocks, const int* q_start, const int* ctx_len,
+                             void* out, int R, int r_prefill, int max_q_len, int max_ctx, int nh, int nkv,
+                             int hd, int bs, float scale, float softcap, int window, int decode_chunk,
+                             void* workspace, size_t workspace_bytes, int mask_chunk, int sink, int wide_weights,
+                             void* stream) {
+  return zk_attention_bf16_maps(q, q_stride, kcache, vcache_t, block_table, max_blocks, q_start, ctx_len, out, R,
+                                r_prefill, max_q_len, max_ctx, nh, nkv, hd, bs, scale, softcap, window, decode_chunk,
+                                workspace, workspace_bytes, mask_chunk, sink, wide_weights, 0, stream);
+}
+
 int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const void* vcache_t,
                       const int* block_table, int max_blocks, const int* q_start, const int* ctx_len,
                       void* out, int R, int r_prefill, int max_q_len, int max_ctx, int nh, int nkv,
@@ -1353,5 +1377,9 @@ extern "C" int zk_steplist_register(const char* name, int nargs, void* fn);
 static const int zk_attention_bf16_masked_entered = zk_steplist_register(
     "zk_attention_bf16_masked", zk_packed::Call<zk_attention_bf16_masked>::nargs,
     (void*)zk_packed::Call<zk_attention_bf16_masked>::call);
+
+static const int zk_attention_bf16_maps_entered = zk_steplist_register(
+    "zk_attention_bf16_maps", zk_packed::Call<zk_attention_bf16_maps>::nargs,
+    (void*)zk_packed::Call<zk_attention_bf16_maps>::call);
 
 #endif  // ZSE_ACT_BF16

@@ -4,7 +4,8 @@
 //   s_m,j = cap tanh((q_m . k_m,j) scale / cap),   a_m = sum_j softmax(s_m)_j v_j,   m = 1, 2
 //   o = a_1 - lambda a_2;   o <- o / sqrt(mean(o^2) + eps) (1 - diff)
 //
-// A key head of the cache holds both maps' keys, [k1 | k2], 2 D channels; its values have E.
+// The cache keeps a key head of D channels per (key/value head, map), head 2 g + m, and one value
+// head of E channels per key/value head g: both maps read the same values.
 // The plain kernel: one wave per (token, query head), keys in tiles of 64 aligned to absolute
 // positions with a running maximum and sum per map, so the order of every sum follows from the
 // token's position alone.  Everything float.  ``zk_cache_store`` copies a step's keys and values
@@ -24,21 +25,21 @@ __device__ __forceinline__ float query_temperature(int pos, float coef, int ever
 
 __global__ __launch_bounds__(256) void cache_store_kernel(const act_t* __restrict__ rows, int ld, int k_off, int v_off,
                                                           const int* __restrict__ slot_map, act_t* __restrict__ kcache,
-                                                          act_t* __restrict__ vcache, int nkv, int hd, int vd, int bs,
+                                                          act_t* __restrict__ vcache, int nk, int hd, int nv, int vd, int bs,
                                                           int v_transposed) {
   const int t = blockIdx.x;
   const int slot = slot_map[t];
   if (slot < 0) return;
   const size_t page = slot / bs, off = slot % bs;
   const act_t* row = rows + (size_t)t * ld;
-  for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) {
+  for (int i = threadIdx.x; i < nk * hd; i += blockDim.x) {
     const int g = i / hd, d = i % hd;
-    kcache[((page * nkv + g) * bs + off) * hd + d] = row[k_off + i];
+    kcache[((page * nk + g) * bs + off) * hd + d] = row[k_off + i];
   }
-  for (int i = threadIdx.x; i < nkv * vd; i += blockDim.x) {
+  for (int i = threadIdx.x; i < nv * vd; i += blockDim.x) {
     const int g = i / vd, d = i % vd;
-    if (v_transposed) vcache[(page * nkv + g) * (size_t)vd * bs + (size_t)d * bs + off] = row[v_off + i];
-    else vcache[((page * nkv + g) * bs + off) * vd + d] = row[v_off + i];
+    if (v_transposed) vcache[(page * nv + g) * (size_t)vd * bs + (size_t)d * bs + off] = row[v_off + i];
+    else vcache[((page * nv + g) * bs + off) * vd + d] = row[v_off + i];
   }
 }
 
@@ -75,11 +76,11 @@ __global__ __launch_bounds__(64) void diff_attention_plain_kernel(
     int page = -1;
     if (valid) {
       page = table[j / bs];
-      const act_t* kr = kcache + (((size_t)page * nkv + kvh) * bs + (j % bs)) * (2 * D);
 #pragma unroll
       for (int mp = 0; mp < 2; mp++) {
+        const act_t* kr = kcache + (((size_t)page * 2 * nkv + 2 * kvh + mp) * bs + (j % bs)) * D;
         float dot = 0.f;
-        for (int d = 0; d < D; d++) dot = fmaf(sq[mp * D + d], to_f32(kr[mp * D + d]), dot);
+        for (int d = 0; d < D; d++) dot = fmaf(sq[mp * D + d], to_f32(kr[d]), dot);
         float x = dot * scale;
         if (softcap > 0.f) x = softcap * tanhf(x / softcap);
         s[mp] = x;
@@ -135,6 +136,19 @@ __global__ __launch_bounds__(64) void diff_attention_plain_kernel(
   }
 }
 
+// q rows times the temperature of their positions, in place (for an attention kernel that takes
+// its queries as they lie)
+__global__ void query_temperature_kernel(act_t* __restrict__ q, int ld, int width, const int* __restrict__ positions,
+                                         float coef, int every) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  if (pos < 0) return;
+  const float c = query_temperature(pos, coef, every);
+  if (c == 1.0f) return;
+  act_t* row = q + (size_t)t * ld;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) row[i] = from_f32<act_t>(to_f32(row[i]) * c);
+}
+
 // Joins two maps' outputs that an ordinary attention kernel computed as heads of their own:
 // a: [T, nh, 2, E] (map 1 then map 2 of each head) -> out [T, nh, E].
 __global__ __launch_bounds__(64) void diff_join_kernel(const act_t* __restrict__ a, act_t* __restrict__ out, int E,
@@ -161,20 +175,21 @@ __global__ __launch_bounds__(64) void diff_join_kernel(const act_t* __restrict__
 
 extern "C" {
 
-// rows: [T, ld]; a row's nkv key heads of hd begin at column k_off, its nkv value heads of vd at v_off.
+// rows: [T, ld]; a row's nk key heads of hd begin at column k_off, its nv value heads of vd at v_off.
+// kcache: [pages, nk, bs, hd]; vcache: [pages, nv, bs, vd], or [pages, nv, vd, bs] when v_transposed.
 int zk_cache_store(const void* rows, int ld, int k_off, int v_off, const int* slot_map, void* kcache, void* vcache, int T,
-                   int nkv, int hd, int vd, int bs, int v_transposed, void* stream) {
-  ZK_REQUIRE(T >= 0 && nkv > 0 && hd > 0 && vd > 0 && bs > 0 && slot_map != nullptr && kcache != nullptr && vcache != nullptr,
+                   int nk, int hd, int nv, int vd, int bs, int v_transposed, void* stream) {
+  ZK_REQUIRE(T >= 0 && nk > 0 && nv > 0 && hd > 0 && vd > 0 && bs > 0 && slot_map != nullptr && kcache != nullptr && vcache != nullptr,
              "zk_cache_store: bad arguments");
-  ZK_REQUIRE(k_off >= 0 && v_off >= 0 && ld >= k_off + nkv * hd && ld >= v_off + nkv * vd, "zk_cache_store: rows shorter than their heads");
+  ZK_REQUIRE(k_off >= 0 && v_off >= 0 && ld >= k_off + nk * hd && ld >= v_off + nv * vd, "zk_cache_store: rows shorter than their heads");
   if (T == 0) return 0;
   cache_store_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)rows, ld, k_off, v_off, slot_map, (act_t*)kcache,
-                                                        (act_t*)vcache, nkv, hd, vd, bs, v_transposed);
+                                                        (act_t*)vcache, nk, hd, nv, vd, bs, v_transposed);
   return zk_launch_status("zk_cache_store");
 }
 
-// q: rows q_stride apart, nh heads of [map 1 | map 2], D channels each; the cache's key heads have
-// 2 D channels, its value heads E; out: [T, nh, E].  softcap <= 0: none; window <= 0: every earlier
+// q: rows q_stride apart, nh heads of [map 1 | map 2], D channels each; the cache holds 2 nkv key
+// heads of D channels (head 2 g + m: map m of key/value head g) and nkv value heads of E; out: [T, nh, E].  softcap <= 0: none; window <= 0: every earlier
 // key; every <= 0: no query temperature.
 int zk_diff_attention_plain(const void* q, int q_stride, const void* kcache, const void* vcache, const int* block_table,
                             int max_blocks, const int* req_of_token, const int* positions, void* out, int T, int nh,
@@ -192,6 +207,14 @@ int zk_diff_attention_plain(const void* q, int q_stride, const void* kcache, con
   return zk_launch_status("zk_diff_attention_plain");
 }
 
+// q: [T, ld], of which the first ``width`` columns are multiplied by 1 + coef ln(floor((p + 1) / every) + 1).
+int zk_query_temperature(void* q, int ld, int width, const int* positions, int T, float coef, int every, void* stream) {
+  ZK_REQUIRE(T >= 0 && width > 0 && ld >= width && every > 0, "zk_query_temperature: bad sizes");
+  if (T == 0) return 0;
+  query_temperature_kernel<<<T, 256, 0, (hipStream_t)stream>>>((act_t*)q, ld, width, positions, coef, every);
+  return zk_launch_status("zk_query_temperature");
+}
+
 // a: [T, nh, 2, E] -> out [T, nh, E]: a1 - lambda a2, unit RMS over E, times (1 - diff).
 int zk_diff_join(const void* a, void* out, int T, int nh, int E, float lambda, float diff, float eps, void* stream) {
   ZK_REQUIRE(T >= 0 && nh > 0 && nh <= 65535 && E > 0 && E <= DA_MAX, "zk_diff_join: bad sizes");
@@ -206,3 +229,4 @@ int zk_diff_join(const void* a, void* out, int T, int nh, int E, float lambda, f
 ZK_ENTER(zk_cache_store)
 ZK_ENTER(zk_diff_attention_plain)
 ZK_ENTER(zk_diff_join)
+ZK_ENTER(zk_query_temperature)

@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
     const __bf16* __restrict__ qa, const __bf16* __restrict__ kcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, const float* __restrict__ sinks,
     __bf16* __restrict__ out, float* __restrict__ part, int H, int HD, int C, int HDP, int bs, float scale, int splits,
-    int split_keys) {
+    int split_keys, int window) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int LDK = HDP + 8;
   __bf16* Ks = (__bf16*)smem;                       // [32][LDK]
@@ -248,10 +248,15 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
   }
   const int wrow = row0 + wave * 32 + lr;
   const int my_pos = wrow < rows ? ctx - n_q + wrow / H : -1;
+  // with a window a row sees the keys [my_lo, my_pos]; the block begins at the tile that holds the
+  // first key of its first row (pages before it may have gone back to the pool: the table names none)
+  const int my_lo = window > 0 ? max(my_pos - window + 1, 0) : 0;
+  const int block_lo = window > 0 ? max(ctx - n_q + row0 / H - window + 1, 0) / 32 * 32 : 0;
   const bool wave_live = row0 + wave * 32 < rows;
   const int last_row = min(rows, row0 + LA_ROWS) - 1;
-  const int k_begin = split * split_keys;
-  const int k_end = min(ctx - n_q + last_row / H + 1, (split + 1) * split_keys);      // exclusive
+  // the ranges of a split count from the block's first tile
+  const int k_begin = block_lo + split * split_keys;
+  const int k_end = min(ctx - n_q + last_row / H + 1, block_lo + (split + 1) * split_keys);      // exclusive
   float m = -INFINITY, l = 0.f;
   floatx16_t o[DT];
 #pragma unroll
@@ -271,7 +276,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
       bf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
       if (i < 32 * pieces && key < k_end && c8 < HD) {
         const int page = table[key / bs];
-        v = *(const bf16x8_t*)(kcache + ((size_t)page * bs + key % bs) * HD + c8);
+        if (page >= 0) v = *(const bf16x8_t*)(kcache + ((size_t)page * bs + key % bs) * HD + c8);
       }
       nxt[u] = v;
     }
@@ -306,7 +311,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
 #pragma unroll
     for (int e = 0; e < 16; e++) {
       const int key = key0 + (e / 4) * 8 + lh * 4 + (e % 4);
-      const bool seen = key <= my_pos && key < k_end;
+      const bool seen = key <= my_pos && key >= my_lo && key < k_end;
       s[e] = seen ? s[e] * scale : -INFINITY;
       mt = fmaxf(mt, s[e]);
     }
@@ -432,10 +437,11 @@ size_t zk_latent_attention_bf16_workspace(int T, int H, int C, int splits) {
 // out: [T, H, C].  Request r holds rows [q_start[r], q_start[r + 1]) and ends at position
 // ctx_len[r] - 1.  max_q_len, max_ctx: the longest portion and context of the step (they size
 // the grid).  work: float scratch of work_bytes (may be null: no ranges).
-int zk_latent_attention_bf16(const void* qa, const void* kcache, const int* block_table, int max_blocks,
-                             const int* q_start, const int* ctx_len, const int* positions, const float* sinks, void* out,
-                             void* work, size_t work_bytes, int T, int R, int max_q_len, int max_ctx, int H, int HD, int C,
-                             int bs, float scale, void* stream) {
+// window > 0: a row at position p sees the keys [max(0, p - window + 1), p] only.
+int zk_latent_attention_bf16_window(const void* qa, const void* kcache, const int* block_table, int max_blocks,
+                                    const int* q_start, const int* ctx_len, const int* positions, const float* sinks,
+                                    void* out, void* work, size_t work_bytes, int T, int R, int max_q_len, int max_ctx, int H,
+                                    int HD, int C, int bs, float scale, int window, void* stream) {
   ZK_REQUIRE(T >= 0 && R >= 0 && H > 0 && max_q_len > 0 && max_ctx > 0 && max_blocks > 0, "zk_latent_attention_bf16: bad sizes");
   ZK_REQUIRE(zk_latent_attention_bf16_supports(HD, C, bs), "zk_latent_attention_bf16: rows of up to 320 channels in eights, up to 256 of them values");
   ZK_REQUIRE(R <= 65535, "zk_latent_attention_bf16: too many requests");
@@ -445,14 +451,17 @@ int zk_latent_attention_bf16(const void* qa, const void* kcache, const int* bloc
   const int groups = (int)(((size_t)max_q_len * H + LA_ROWS - 1) / LA_ROWS);
   int splits = 1;
   const int blocks = groups * R;
+  // the keys a block walks: with a window, those of its rows' windows (and the tile they begin in)
+  const int keys = window > 0 ? min(max_ctx, window + (LA_ROWS + H - 1) / H + 32) : max_ctx;
   if (blocks < 128 && work != nullptr) {
+    // (with a window, ranges that lie before it are empty: only those over the window's keys count)
     splits = (256 + blocks - 1) / blocks;
-    splits = min(splits, (max_ctx + 127) / 128);
+    splits = min(splits, (keys + 127) / 128);
     splits = min(splits, 64);
     while (splits > 1 && zk_latent_attention_bf16_workspace(T, H, C, splits) > work_bytes) splits--;
     splits = max(splits, 1);
   }
-  const int split_keys = splits == 1 ? 0x40000000 : ((max_ctx + splits - 1) / splits + 31) / 32 * 32;
+  const int split_keys = splits == 1 ? 0x40000000 : ((keys + splits - 1) / splits + 31) / 32 * 32;
   const size_t lds = ((size_t)32 * (HDP + 8) + (size_t)DT * 32 * LA_VT_LD + (size_t)LA_ROWS * (HDP + 8)) * sizeof(__bf16);
   dim3 grid(groups, R, splits);
   hipStream_t st = (hipStream_t)stream;
@@ -465,7 +474,7 @@ int zk_latent_attention_bf16(const void* qa, const void* kcache, const int* bloc
     }                                                                                                                  \
     latent_attn_kernel<N><<<grid, 256, lds, st>>>((const __bf16*)qa, (const __bf16*)kcache, block_table, max_blocks,   \
                                                   q_start, ctx_len, sinks, (__bf16*)out, (float*)work, H, HD, C, HDP,  \
-                                                  bs, scale, splits, split_keys);                                      \
+                                                  bs, scale, splits, split_keys, window);                              \
   } while (0)
   if (DT == 2) LA_LAUNCH(2);
   else if (DT == 4) LA_LAUNCH(4);
@@ -476,7 +485,16 @@ int zk_latent_attention_bf16(const void* qa, const void* kcache, const int* bloc
   return zk_launch_status("zk_latent_attention_bf16");
 }
 
+int zk_latent_attention_bf16(const void* qa, const void* kcache, const int* block_table, int max_blocks,
+                             const int* q_start, const int* ctx_len, const int* positions, const float* sinks, void* out,
+                             void* work, size_t work_bytes, int T, int R, int max_q_len, int max_ctx, int H, int HD, int C,
+                             int bs, float scale, void* stream) {
+  return zk_latent_attention_bf16_window(qa, kcache, block_table, max_blocks, q_start, ctx_len, positions, sinks, out, work,
+                                         work_bytes, T, R, max_q_len, max_ctx, H, HD, C, bs, scale, 0, stream);
+}
+
 }  // extern "C"
 
 ZK_ENTER(zk_latent_attention_bf16)
+ZK_ENTER(zk_latent_attention_bf16_window)
 #endif

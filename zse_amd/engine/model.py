@@ -106,7 +106,8 @@ class Model:
             if isinstance(need, PagedKV):
                 seen = min(context, need.window) if need.window else context
                 vd = 0 if getattr(need, "values_in_keys", False) else (need.value_dim or need.head_dim)
-                total += need.num_kv_heads * (need.head_dim + vd) * seen * itemsize
+                nv = getattr(need, "value_heads", None) or need.num_kv_heads
+                total += (need.num_kv_heads * need.head_dim + nv * vd) * seen * itemsize
         return total
 
     @staticmethod

@@ -192,9 +192,10 @@ class StepRunner:
                 cc.v_transposed = bool(self.tuned and getattr(mixer, "wants_v_transposed", None) and
                                        mixer.wants_v_transposed(self.k, self.dtype, self.page_size))
                 vd = need.value_dim or need.head_dim
-                shape = (pages, need.num_kv_heads, self.page_size, vd)
+                nv = getattr(need, "value_heads", None) or need.num_kv_heads
+                shape = (pages, nv, self.page_size, vd)
                 if cc.v_transposed:
-                    shape = (pages, need.num_kv_heads, vd, self.page_size)
+                    shape = (pages, nv, vd, self.page_size)
                 # values that are part of the keys have no slab of their own
                 cc.v = cc.k if getattr(need, "values_in_keys", False) else rt.zeros(shape, self.dtype)
                 if getattr(need, "state_bytes", 0):      # a mixer that keeps a state beside its pages

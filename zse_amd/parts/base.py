@@ -54,6 +54,8 @@ class PagedKV:
     values_in_keys: bool = False        # a value is the first value_dim channels of its key: no value slab is kept
     chunk: Optional[int] = None
     state_bytes: int = 0
+    value_heads: Optional[int] = None   # value heads where they are fewer than the key heads (several maps of keys
+    #                                     over the same values); None: as many
 
 
 @dataclass(frozen=True)

@@ -91,7 +91,7 @@ class LatentAttention(Part):
     def _fast(self, kernels, dtype: str, page_size: int) -> bool:
         """Whether the matrix-core attention kernel serves this layer."""
         s = self.spec
-        return bool(dtype == BF16 and not s.window and kernels.has("zk_latent_attention_bf16") and
+        return bool(dtype == BF16 and kernels.has("zk_latent_attention_bf16_window") and
                     kernels.zk_latent_attention_bf16_supports(s.latent_dim + s.rotary_dim, s.latent_dim, page_size))
 
     def prepare(self, kernels, dtype, max_seqs, max_model_len, page_size, max_batch_tokens=0) -> int:
@@ -137,10 +137,10 @@ class LatentAttention(Part):
         o = ctx.alloc((T, H * C))
         sinks = self.sinks.ptr if self.sinks is not None else None
         if ctx.tuned and self._fast(k, ctx.dtype, g.page_size):
-            k.zk_latent_attention_bf16(qa.ptr, cache.k.ptr, g.block_table, g.max_blocks, ctx.q_start, ctx.ctx_len,
-                                       ctx.positions, sinks, o.ptr, ctx.workspace.ptr, ctx.workspace.nbytes, T, ctx.R,
-                                       max(int(ctx.max_q_len), 1), int(ctx.max_ctx), H, C + R, C, g.page_size,
-                                       float(s.scale), ctx.stream)
+            k.zk_latent_attention_bf16_window(qa.ptr, cache.k.ptr, g.block_table, g.max_blocks, ctx.q_start, ctx.ctx_len,
+                                              ctx.positions, sinks, o.ptr, ctx.workspace.ptr, ctx.workspace.nbytes, T, ctx.R,
+                                              max(int(ctx.max_q_len), 1), int(ctx.max_ctx), H, C + R, C, g.page_size,
+                                              float(s.scale), int(s.window) if s.window else 0, ctx.stream)
         else:
             k.zk_attention_plain_sink(qa.ptr, H * (C + R), cache.k.ptr, cache.k.ptr, g.block_table, g.max_blocks,
                                       ctx.req_of_token, ctx.positions, o.ptr, T, H, 1, C + R, C, g.page_size,

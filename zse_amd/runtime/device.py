@@ -214,7 +214,8 @@ KERNEL_SIGNATURES = {
     "zk_moe_route_ext": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP],
     "zk_moe_experts_ext": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _VP],
     "zk_gate_rows": [_VP, _VP, _I, _I, _I, _VP],
-    "zk_cache_store": [_VP, _I, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_cache_store": [_VP, _I, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_query_temperature": [_VP, _I, _I, _VP, _I, _F, _I, _VP],
     "zk_diff_attention_plain": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I,
                                 _F, _F, _F, _F, _I, _VP],
     "zk_diff_join": [_VP, _VP, _I, _I, _I, _F, _F, _F, _VP],
@@ -235,6 +236,10 @@ BF16_KERNEL_SIGNATURES = {
                                  _F, _F, _I, _I, _VP, _SZ, _I, _I, _I, _VP],
     "zk_latent_attention_bf16": [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _SZ, _I, _I, _I, _I, _I, _I, _I, _I, _F, _VP],
     "zk_moe_experts_grouped": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP],
+    "zk_attention_bf16_maps": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
+                               _F, _F, _I, _I, _VP, _SZ, _I, _I, _I, _I, _VP],
+    "zk_latent_attention_bf16_window": [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _SZ, _I, _I, _I, _I, _I, _I, _I, _I, _F,
+                                        _I, _VP],
     "zk_moe_experts_grouped_ext": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _VP],
 }
 
