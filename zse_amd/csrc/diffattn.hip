@@ -26,8 +26,18 @@ __device__ __forceinline__ float query_temperature(int pos, float coef, int ever
 __global__ __launch_bounds__(256) void cache_store_kernel(const act_t* __restrict__ rows, int ld, int k_off, int v_off,
                                                           const int* __restrict__ slot_map, act_t* __restrict__ kcache,
                                                           act_t* __restrict__ vcache, int nk, int hd, int nv, int vd, int bs,
-                                                          int v_transposed) {
+                                                          int v_transposed, act_t* __restrict__ q, int q_width,
+                                                          const int* __restrict__ positions, float coef, int every) {
   const int t = blockIdx.x;
+  if (q != nullptr) {
+    // the queries of the row times the temperature of its position, in place
+    const int pos = positions[t];
+    const float c = pos >= 0 ? query_temperature(pos, coef, every) : 1.0f;
+    if (c != 1.0f) {
+      act_t* qr = q + (size_t)t * ld;
+      for (int i = threadIdx.x; i < q_width; i += blockDim.x) qr[i] = from_f32<act_t>(to_f32(qr[i]) * c);
+    }
+  }
   const int slot = slot_map[t];
   if (slot < 0) return;
   const size_t page = slot / bs, off = slot % bs;
@@ -184,7 +194,24 @@ int zk_cache_store(const void* rows, int ld, int k_off, int v_off, const int* sl
   ZK_REQUIRE(k_off >= 0 && v_off >= 0 && ld >= k_off + nk * hd && ld >= v_off + nv * vd, "zk_cache_store: rows shorter than their heads");
   if (T == 0) return 0;
   cache_store_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)rows, ld, k_off, v_off, slot_map, (act_t*)kcache,
-                                                        (act_t*)vcache, nk, hd, nv, vd, bs, v_transposed);
+                                                        (act_t*)vcache, nk, hd, nv, vd, bs, v_transposed, nullptr, 0, nullptr,
+                                                        0.f, 0);
+  return zk_launch_status("zk_cache_store");
+}
+
+// The same, and the first q_width columns of every row (the queries) times the temperature of the
+// row's position, 1 + coef ln(floor((p + 1) / every) + 1), in place: one launch for both.
+int zk_cache_store_temperature(void* rows, int ld, int q_width, int k_off, int v_off, const int* positions,
+                               const int* slot_map, void* kcache, void* vcache, int T, int nk, int hd, int nv, int vd, int bs,
+                               int v_transposed, float coef, int every, void* stream) {
+  ZK_REQUIRE(T >= 0 && nk > 0 && nv > 0 && hd > 0 && vd > 0 && bs > 0 && slot_map != nullptr && kcache != nullptr && vcache != nullptr,
+             "zk_cache_store: bad arguments");
+  ZK_REQUIRE(k_off >= q_width && v_off >= q_width && ld >= k_off + nk * hd && ld >= v_off + nv * vd && q_width > 0 && every > 0 &&
+             positions != nullptr, "zk_cache_store: rows shorter than their heads, or queries that overlap them");
+  if (T == 0) return 0;
+  cache_store_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)rows, ld, k_off, v_off, slot_map, (act_t*)kcache,
+                                                        (act_t*)vcache, nk, hd, nv, vd, bs, v_transposed, (act_t*)rows, q_width,
+                                                        positions, coef, every);
   return zk_launch_status("zk_cache_store");
 }
 
@@ -227,6 +254,7 @@ int zk_diff_join(const void* a, void* out, int T, int nh, int E, float lambda, f
 }  // extern "C"
 
 ZK_ENTER(zk_cache_store)
+ZK_ENTER(zk_cache_store_temperature)
 ZK_ENTER(zk_diff_attention_plain)
 ZK_ENTER(zk_diff_join)
 ZK_ENTER(zk_query_temperature)

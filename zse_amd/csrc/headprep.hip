@@ -153,22 +153,22 @@ extern "C" int zk_head_prep(void* qkv, const int* positions, const int* slot_map
 //
 // One block per token: a row holds nh query heads, then nkv key heads of D (and, without
 // values_are_keys, nkv value heads of E that are stored as they are).  Float throughout, one
-// rounding at the store.  The block is 256 wide whatever the step, so a row's sums do not
-// depend on what else the step holds.
-__global__ __launch_bounds__(256) void row_prep_kernel(
+// rounding at the store.  In the 32-bit library the block is 256 wide whatever the step, so a row's
+// sums do not depend on what else the step holds; in bfloat16 steps of up to 64 rows take 1,024 threads a row.
+__global__ __launch_bounds__(1024) void row_prep_kernel(
     act_t* __restrict__ qk, int ld, const int* __restrict__ positions, const int* __restrict__ slot_map,
     const float* __restrict__ bias, const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
     const float* __restrict__ inv_freq, int rot_dims, act_t* __restrict__ kcache, act_t* __restrict__ vcache, int nh,
     int nkv, int D, int E, int bs, int v_transposed, int values_are_keys) {
   extern __shared__ float row[];                 // [(nh + nkv) D]
   __shared__ float red[17];
-  const int t = blockIdx.x, tid = threadIdx.x;
+  const int t = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
   const int pos = positions[t];
   if (pos < 0) return;
   const int nq = nh * D, nk = nkv * D;
   act_t* src = qk + (size_t)t * ld;
   float sq = 0.f, sk = 0.f;
-  for (int i = tid; i < nq + nk; i += 256) {
+  for (int i = tid; i < nq + nk; i += nt) {
     float x = to_f32(src[i]);
     if (bias) x += bias[i];
     row[i] = x;
@@ -182,7 +182,7 @@ __global__ __launch_bounds__(256) void row_prep_kernel(
   if (slot >= 0) {
     // the values: the keys before norm and rotation, or the row's own value heads
     const int nv = nkv * E;
-    for (int i = tid; i < nv; i += 256) {
+    for (int i = tid; i < nv; i += nt) {
       const int g = i / E, d = i % E;
       float x;
       if (values_are_keys) x = row[nq + i];
@@ -197,16 +197,16 @@ __global__ __launch_bounds__(256) void row_prep_kernel(
   __syncthreads();
   if (q_gain) {
     const float inv = 1.0f / sqrtf(sq / (float)nq + eps);
-    for (int i = tid; i < nq; i += 256) row[i] = row[i] * inv * q_gain[i];
+    for (int i = tid; i < nq; i += nt) row[i] = row[i] * inv * q_gain[i];
   }
   if (k_gain) {
     const float inv = 1.0f / sqrtf(sk / (float)nk + eps);
-    for (int i = tid; i < nk; i += 256) row[nq + i] = row[nq + i] * inv * k_gain[i];
+    for (int i = tid; i < nk; i += nt) row[nq + i] = row[nq + i] * inv * k_gain[i];
   }
   __syncthreads();
   if (inv_freq) {
     const int half = rot_dims / 2;
-    for (int i = tid; i < (nh + nkv) * half; i += 256) {
+    for (int i = tid; i < (nh + nkv) * half; i += nt) {
       const int head = i / half, m = i % half;
       float sn, cs, ra, rb;
       sincosf((float)pos * inv_freq[m], &sn, &cs);
@@ -217,9 +217,9 @@ __global__ __launch_bounds__(256) void row_prep_kernel(
     }
     __syncthreads();
   }
-  for (int i = tid; i < nq; i += 256) src[i] = from_f32<act_t>(row[i]);
+  for (int i = tid; i < nq; i += nt) src[i] = from_f32<act_t>(row[i]);
   if (slot >= 0)
-    for (int i = tid; i < nk; i += 256) {
+    for (int i = tid; i < nk; i += nt) {
       const int g = i / D, d = i % D;
       kcache[((page * nkv + g) * bs + off) * D + d] = from_f32<act_t>(row[nq + i]);
     }
@@ -246,7 +246,8 @@ extern "C" int zk_row_prep(void* qk, int ld, const int* positions, const int* sl
     hipFuncSetAttribute((const void*)row_prep_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
     raised = true;
   }
-  row_prep_kernel<<<T, 256, lds, (hipStream_t)stream>>>((act_t*)qk, ld, positions, slot_map, bias, q_gain, k_gain, eps,
+  const int threads = (ZSE_ACT_BF16 && T <= 64) ? 1024 : 256;
+  row_prep_kernel<<<T, threads, lds, (hipStream_t)stream>>>((act_t*)qk, ld, positions, slot_map, bias, q_gain, k_gain, eps,
                                                        inv_freq, rot_dims, (act_t*)kcache, (act_t*)vcache, nh, nkv, D, E,
                                                        bs, v_transposed, values_are_keys);
   return zk_launch_status("zk_row_prep");

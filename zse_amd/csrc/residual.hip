@@ -157,8 +157,11 @@ int zk_sum_layer_norm(float* h, const void* a, int a_parts, const void* b, int b
   ZK_REQUIRE(T >= 0 && W > 0 && a_parts >= 0 && b_parts >= 0, "zk_sum_layer_norm: bad sizes");
   ZK_REQUIRE(w_next == nullptr || out != nullptr, "zk_sum_layer_norm: a norm without output");
   if (T == 0) return 0;
-  sum_layer_norm_kernel<<<T, 256, 0, (hipStream_t)stream>>>(h, a, a_parts, b, b_parts, bias, w_next, c_next, eps,
-                                                           (act_t*)out, W);
+  // (in the 32-bit library the block is always 256 wide: the order of a row's sums must not follow
+  // from how many rows a step brings)
+  const int threads = (ZSE_ACT_BF16 && T <= 64 && W >= 1024) ? 1024 : 256;
+  sum_layer_norm_kernel<<<T, threads, 0, (hipStream_t)stream>>>(h, a, a_parts, b, b_parts, bias, w_next, c_next, eps,
+                                                               (act_t*)out, W);
   return zk_launch_status("zk_sum_layer_norm");
 }
 

@@ -97,14 +97,18 @@ class DifferentialAttention(Part):
         width = (H + G) * 2 * D + G * E
         g = ctx.group(cache.group)
         qkv = linear(ctx, x, self.w_qkv, ctx.alloc((T, width)))
-        k.zk_cache_store(qkv.ptr, width, H * 2 * D, (H + G) * 2 * D, g.slot_map, cache.k.ptr, cache.v.ptr, T, 2 * G, D, G, E,
-                         g.page_size, 1 if cache.v_transposed else 0, ctx.stream)
+        fast = bool(cache.v_transposed and ctx.tuned)
+        store = (g.slot_map, cache.k.ptr, cache.v.ptr, T, 2 * G, D, G, E, g.page_size, 1 if cache.v_transposed else 0)
+        if fast and s.temp_every > 0:
+            # the matrix-core kernel takes its queries as they lie: the temperature in the storing launch
+            k.zk_cache_store_temperature(qkv.ptr, width, H * 2 * D, H * 2 * D, (H + G) * 2 * D, ctx.positions, *store,
+                                         float(s.temp_coef), int(s.temp_every), ctx.stream)
+        else:
+            k.zk_cache_store(qkv.ptr, width, H * 2 * D, (H + G) * 2 * D, *store, ctx.stream)
         o = ctx.alloc((T, H * E))
         cap, win = float(s.softcap) if s.softcap else 0.0, int(s.window) if s.window else 0
-        if cache.v_transposed and ctx.tuned:
+        if fast:
             # the 2 H maps as heads of the matrix-core kernel; a pair of key heads shares a value head
-            if s.temp_every > 0:
-                k.zk_query_temperature(qkv.ptr, width, H * 2 * D, ctx.positions, T, float(s.temp_coef), int(s.temp_every), ctx.stream)
             maps = ctx.alloc((T, 2 * H * E))
             k.zk_attention_bf16_maps(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks, ctx.q_start,
                                      ctx.ctx_len, maps.ptr, ctx.R, ctx.n_multi, ctx.max_q_len, ctx.max_ctx, 2 * H, 2 * G, D,

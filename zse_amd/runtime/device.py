@@ -215,6 +215,7 @@ KERNEL_SIGNATURES = {
     "zk_moe_experts_ext": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _VP],
     "zk_gate_rows": [_VP, _VP, _I, _I, _I, _VP],
     "zk_cache_store": [_VP, _I, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_cache_store_temperature": [_VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
     "zk_query_temperature": [_VP, _I, _I, _VP, _I, _F, _I, _VP],
     "zk_diff_attention_plain": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I,
                                 _F, _F, _F, _F, _I, _VP],
