@@ -58,7 +58,7 @@ def close(got, want, tol=2e-5):
     assert np.abs(got - want).max() <= tol * max(1.0, np.abs(want).max()), np.abs(got - want).max()
 
 
-@pytest.mark.parametrize("buckets,mp,mc", [(61, 7, 3), (1, 1, 1), (509, 65521, 40503)])
+@pytest.mark.parametrize("buckets,mp,mc", [(61, 7, 3), (1, 1, 1), (509, 65521, 40503), (97, -5, 2)])
 def test_pair_rows_and_the_previous_token(dev, buckets, mp, mc):
     """Two requests whose tokens come in portions of unequal sizes, single tokens among them: the
     token before a portion's first one comes from the request's slot, and the slot's other words

@@ -146,7 +146,6 @@ class RotalornConfig:
             vals = [need(bg, key, int, p, required=True) for key in ("buckets", "mul_prev", "mul_cur")]
             if None not in vals:
                 p.require(vals[0] >= 1, f"embedding.bigram.buckets must be at least 1, got {vals[0]}")
-                p.require(vals[1] >= 0 and vals[2] >= 0, f"embedding.bigram: multipliers must not be negative, got {vals[1:]}")
                 bigram = tuple(vals)
         p.raise_if_any()
         p.require(V > 0 and W > 0, f"'vocab' and 'width' must be positive, got {V} and {W}")
