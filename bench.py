@@ -509,14 +509,14 @@ def rotalorn_config(width, heads, kv_heads, dim, ff, groups, vocab, window):
             {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
                                             "mask": {"size": window},
                                             "rot": {"base": 10000.0, "dims": dim // 2,
-                                                    "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 2048}}},
+                                                    "scaling": {"factor": 4.0, "low": 1.0, "high": 8.0, "original": 2048}}},
              "mlp": dict(moe)},
             {"type": "latent_attention", "mixer": {"heads": heads, "dim": dim // 2, "rot_dim": dim // 4, "vdim": dim // 2,
                                                    "kv_rank": 2 * dim, "q_rank": width // 2, "scale": (3 * dim // 4) ** -0.5,
                                                    "mask": {"size": window}, "rot": {"base": 10000.0, "dims": dim // 4}},
              "mlp": dict(moe)}]
     return {"architecture": "Rotalorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
-            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}}, "layers": layers}
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 8191, "mul_cur": 131}}, "layers": layers}
 
 
 # what is timed, beside which relative, against which plain implementation it is checked first, and

@@ -61,7 +61,7 @@ def config(layers, vocab=96, width=32, eps=1e-5, bigram=(61, 7, 3)):
 CFG_A = config([
     latent_layer(heads=3, dim=8, rot_dim=4, vdim=12, kv_rank=20, q_rank=16, base=3000.0, window=13, mlp=dense(40)),
     diff_layer(heads=4, kv_heads=2, dim=12, vdim=24, diff=0.4, softcap=15.0, q_temp=(0.5, 16), mlp=moe(5, 2, 24, 40)),
-    attention_layer(heads=4, kv_heads=2, dim=24, rot_dims=12, base=500.0, scaling=(8.0, 1.0, 4.0, 64), scale=0.3, window=21,
+    attention_layer(heads=4, kv_heads=2, dim=24, rot_dims=12, base=500.0, scaling=(6.0, 1.0, 3.0, 64), scale=0.3, window=21,
                     mlp=moe(4, 3, 16, 24)),
     diff_layer(heads=2, kv_heads=2, dim=8, vdim=8, diff=0.7, softcap=None, q_temp=(1.5, 5), mlp=dense(56)),
 ], vocab=200, width=48, eps=1e-5, bigram=(61, 7, 3))

@@ -54,7 +54,7 @@ def test_every_constant_comes_from_the_config():
     assert (d.diff, d.softcap, d.temp_coef, d.temp_every, d.scale) == (0.4, 15.0, 0.5, 16, 12 ** -0.5)
     assert plan.layers[3].mixer.softcap is None and plan.layers[3].mixer.temp_every == 5
     a = plan.layers[2].mixer
-    assert a.values_are_keys and a.scale == 0.3 and a.position.wavelength_scaling == (8.0, 1.0, 4.0, 64.0)
+    assert a.values_are_keys and a.scale == 0.3 and a.position.wavelength_scaling == (6.0, 1.0, 3.0, 64.0)
     assert a.position.rotary_dim == 12 and a.norm_eps == 1e-5
     f = plan.layers[1].ffn
     assert (f.scoring, f.scale_input, f.activation, f.top_k, f.num_experts) == ("softmax", False, "silu", 2, 5)
@@ -66,8 +66,8 @@ def test_every_constant_comes_from_the_config():
     assert b.layers[1].ffn is None and b.layers[0].ffn.shared is None and b.layers[0].ffn.shared_gate is None
 
 
-@pytest.mark.parametrize("dims,base,scaling", [(12, 500.0, (8.0, 1.0, 4.0, 64)), (16, 50.0, (4.0, 1.0, 2.0, 32)),
-                                               (4, 10.0, (2.0, 1.0, 4.0, 16)), (64, 1e6, (8.0, 1.0, 4.0, 1024)),
+@pytest.mark.parametrize("dims,base,scaling", [(12, 500.0, (6.0, 1.0, 3.0, 64)), (16, 50.0, (4.0, 1.0, 2.0, 32)),
+                                               (4, 10.0, (2.0, 1.0, 4.0, 16)), (64, 5e5, (6.0, 1.0, 3.0, 512)),
                                                (32, 1e4, None)])
 def test_frequencies_scaled_by_their_wavelengths(dims, base, scaling):
     part = Rotary(RotarySpec(head_dim=dims, rotary_dim=dims, theta=base, wavelength_scaling=scaling))
