@@ -139,6 +139,7 @@ class LatentAttentionSpec:
     # ``names["q"]`` is then [heads * (head_dim + rotary_dim), query_latent_dim]
     query_latent_dim: Optional[int] = None
     # names["gate"]: [num_heads, hidden]; head h's output times sigmoid(W_gate x)_h, one number a head
+    wide_weights: bool = False       # as AttentionSpec.wide_weights
 
 
 @dataclass(frozen=True)
@@ -164,6 +165,7 @@ class DifferentialAttentionSpec:
     temp_every: int
     names: Dict[str, str]            # roles q, k, v, o, lq1, lk1, lq2, lk2
     kind: str = "differential_attention"
+    wide_weights: bool = False       # as AttentionSpec.wide_weights
 
 
 @dataclass(frozen=True)

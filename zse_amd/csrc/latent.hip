@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
     const __bf16* __restrict__ qa, const __bf16* __restrict__ kcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, const float* __restrict__ sinks,
     __bf16* __restrict__ out, float* __restrict__ part, int H, int HD, int C, int HDP, int bs, float scale, int splits,
-    int split_keys, int window) {
+    int split_keys, int window, int wide) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int LDK = HDP + 8;
   __bf16* Ks = (__bf16*)smem;                       // [32][LDK]
@@ -327,11 +327,19 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
     ps += __shfl_xor(ps, 32, 64);
     l = l * corr + ps;
     m = m_new;
-    bf16x8_t pb0, pb1;
+    bf16x8_t pb0, pb1, pr0, pr1;
 #pragma unroll
     for (int e = 0; e < 8; e++) {
       pb0[e] = (__bf16)p[e];
       pb1[e] = (__bf16)p[8 + e];
+    }
+    if (wide) {
+      // a weight meets the values as two bfloat16 numbers: its rounded value and what the rounding left
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        pr0[e] = (__bf16)(p[e] - (float)pb0[e]);
+        pr1[e] = (__bf16)(p[8 + e] - (float)pb1[e]);
+      }
     }
 #pragma unroll
     for (int dt = 0; dt < DT; dt++) {
@@ -350,6 +358,10 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
       }
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb0, o[dt], 0, 0, 0);
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vb, pb1, o[dt], 0, 0, 0);
+      if (wide) {
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pr0, o[dt], 0, 0, 0);
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vb, pr1, o[dt], 0, 0, 0);
+      }
     }
   }
   if (!wave_live || wrow >= rows) return;
@@ -437,11 +449,12 @@ size_t zk_latent_attention_bf16_workspace(int T, int H, int C, int splits) {
 // out: [T, H, C].  Request r holds rows [q_start[r], q_start[r + 1]) and ends at position
 // ctx_len[r] - 1.  max_q_len, max_ctx: the longest portion and context of the step (they size
 // the grid).  work: float scratch of work_bytes (may be null: no ranges).
-// window > 0: a row at position p sees the keys [max(0, p - window + 1), p] only.
+// window > 0: a row at position p sees the keys [max(0, p - window + 1), p] only.  wide: the softmax's
+// weights keep 16 bits of mantissa in the product with the values (two bfloat16 numbers a weight).
 int zk_latent_attention_bf16_window(const void* qa, const void* kcache, const int* block_table, int max_blocks,
                                     const int* q_start, const int* ctx_len, const int* positions, const float* sinks,
                                     void* out, void* work, size_t work_bytes, int T, int R, int max_q_len, int max_ctx, int H,
-                                    int HD, int C, int bs, float scale, int window, void* stream) {
+                                    int HD, int C, int bs, float scale, int window, int wide, void* stream) {
   ZK_REQUIRE(T >= 0 && R >= 0 && H > 0 && max_q_len > 0 && max_ctx > 0 && max_blocks > 0, "zk_latent_attention_bf16: bad sizes");
   ZK_REQUIRE(zk_latent_attention_bf16_supports(HD, C, bs), "zk_latent_attention_bf16: rows of up to 320 channels in eights, up to 256 of them values");
   ZK_REQUIRE(R <= 65535, "zk_latent_attention_bf16: too many requests");
@@ -474,7 +487,7 @@ int zk_latent_attention_bf16_window(const void* qa, const void* kcache, const in
     }                                                                                                                  \
     latent_attn_kernel<N><<<grid, 256, lds, st>>>((const __bf16*)qa, (const __bf16*)kcache, block_table, max_blocks,   \
                                                   q_start, ctx_len, sinks, (__bf16*)out, (float*)work, H, HD, C, HDP,  \
-                                                  bs, scale, splits, split_keys, window);                              \
+                                                  bs, scale, splits, split_keys, window, wide);                        \
   } while (0)
   if (DT == 2) LA_LAUNCH(2);
   else if (DT == 4) LA_LAUNCH(4);
@@ -490,7 +503,7 @@ int zk_latent_attention_bf16(const void* qa, const void* kcache, const int* bloc
                              void* work, size_t work_bytes, int T, int R, int max_q_len, int max_ctx, int H, int HD, int C,
                              int bs, float scale, void* stream) {
   return zk_latent_attention_bf16_window(qa, kcache, block_table, max_blocks, q_start, ctx_len, positions, sinks, out, work,
-                                         work_bytes, T, R, max_q_len, max_ctx, H, HD, C, bs, scale, 0, stream);
+                                         work_bytes, T, R, max_q_len, max_ctx, H, HD, C, bs, scale, 0, 0, stream);
 }
 
 }  // extern "C"

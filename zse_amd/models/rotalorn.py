@@ -40,6 +40,9 @@ from ..config.plan import (AttentionSpec, BlockSpec, DifferentialAttentionSpec, 
 
 NAME = "Rotalorn"
 MAX_POSITION = 1 << 16        # the config names no longest sequence; tables and pools follow the runner's own limits
+# the softmax's weights are 32-bit numbers of the design: where a matrix-core kernel multiplies them with
+# the values they go in as two bfloat16 halves (16 bits of mantissa), not rounded to one
+WIDE_WEIGHTS = True
 DENSE_ACTIVATION = "gelu_tanh"
 EXPERT_ACTIVATION = "silu"
 TYPES = ("attention", "latent_attention", "attention_2")
@@ -239,7 +242,7 @@ def rotalorn_plan(c: RotalornConfig) -> ModelPlan:
                 hidden_size=c.width, num_heads=l.heads, num_kv_heads=l.kv_heads, head_dim=l.dim, scale=l.scale,
                 softcap=None, window=l.window, position=rotary, names={r: mix + r for r in ("q", "k", "o")},
                 biases={r: f"{mix}{r}.b" for r in ("q", "k")}, norm_eps=c.eps,
-                q_row_norm=mix + "q.norm", k_row_norm=mix + "k.norm", values_are_keys=True)
+                q_row_norm=mix + "q.norm", k_row_norm=mix + "k.norm", values_are_keys=True, wide_weights=WIDE_WEIGHTS)
         elif l.type == "latent_attention":
             mixer = LatentAttentionSpec(
                 hidden_size=c.width, num_heads=l.heads, head_dim=l.dim, rotary_dim=l.rot_dim, value_dim=l.vdim,
@@ -249,13 +252,13 @@ def rotalorn_plan(c: RotalornConfig) -> ModelPlan:
                 names={"q": mix + "uq", "q_down": mix + "dq", "q_down_norm": mix + "dq.norm", "down": mix + "dkv",
                        "down_norm": mix + "dkv.norm", "up_k": mix + "uk", "up_v": mix + "uv", "gate": mix + "g",
                        "o": mix + "o"},
-                window=l.window, query_latent_dim=l.q_rank)
+                window=l.window, query_latent_dim=l.q_rank, wide_weights=WIDE_WEIGHTS)
         else:
             mixer = DifferentialAttentionSpec(
                 hidden_size=c.width, num_heads=l.heads, num_kv_heads=l.kv_heads, head_dim=l.dim, value_dim=l.vdim,
                 scale=l.scale, softcap=l.softcap, window=l.window, diff=l.diff, eps=c.eps, temp_coef=l.temp_coef,
                 temp_every=l.temp_every,
-                names={r: mix + r for r in ("q", "k", "v", "o", "lq1", "lk1", "lq2", "lk2")})
+                names={r: mix + r for r in ("q", "k", "v", "o", "lq1", "lk1", "lq2", "lk2")}, wide_weights=WIDE_WEIGHTS)
         ffn = None
         if l.mlp is not None and l.mlp.kind == "dense":
             ffn = GatedMLPSpec(hidden_size=c.width, intermediate_size=l.mlp.ff, activation=DENSE_ACTIVATION,

@@ -113,7 +113,7 @@ class DifferentialAttention(Part):
             k.zk_attention_bf16_maps(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks, ctx.q_start,
                                      ctx.ctx_len, maps.ptr, ctx.R, ctx.n_multi, ctx.max_q_len, ctx.max_ctx, 2 * H, 2 * G, D,
                                      g.page_size, float(s.scale), cap, win, self.decode_chunk, ctx.workspace.ptr,
-                                     ctx.workspace.nbytes, 0, 0, 0, 1, ctx.stream)
+                                     ctx.workspace.nbytes, 0, 0, 1 if getattr(s, "wide_weights", False) else 0, 1, ctx.stream)
             k.zk_diff_join(maps.ptr, o.ptr, T, H, E, float(self.lam), float(s.diff), float(s.eps), ctx.stream)
             return linear(ctx, o, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)
         k.zk_diff_attention_plain(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks, ctx.req_of_token,

@@ -140,7 +140,8 @@ class LatentAttention(Part):
             k.zk_latent_attention_bf16_window(qa.ptr, cache.k.ptr, g.block_table, g.max_blocks, ctx.q_start, ctx.ctx_len,
                                               ctx.positions, sinks, o.ptr, ctx.workspace.ptr, ctx.workspace.nbytes, T, ctx.R,
                                               max(int(ctx.max_q_len), 1), int(ctx.max_ctx), H, C + R, C, g.page_size,
-                                              float(s.scale), int(s.window) if s.window else 0, ctx.stream)
+                                              float(s.scale), int(s.window) if s.window else 0,
+                                              1 if getattr(s, "wide_weights", False) else 0, ctx.stream)
         else:
             k.zk_attention_plain_sink(qa.ptr, H * (C + R), cache.k.ptr, cache.k.ptr, g.block_table, g.max_blocks,
                                       ctx.req_of_token, ctx.positions, o.ptr, T, H, 1, C + R, C, g.page_size,

@@ -240,7 +240,7 @@ BF16_KERNEL_SIGNATURES = {
     "zk_attention_bf16_maps": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
                                _F, _F, _I, _I, _VP, _SZ, _I, _I, _I, _I, _VP],
     "zk_latent_attention_bf16_window": [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _SZ, _I, _I, _I, _I, _I, _I, _I, _I, _F,
-                                        _I, _VP],
+                                        _I, _I, _VP],
     "zk_moe_experts_grouped_ext": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _VP],
 }
 
